@@ -1,0 +1,221 @@
+// Gated DeltaNet single-token decode: one recurrent step per (request, value head).
+//
+//   S <- g*S;  u = S^T k;  delta = beta*(v - u);  S <- S + k delta^T;  o = S^T q * dk^-1/2
+//
+// with S the fp32 [dk, dv] state of the head (row-major, dv contiguous), q/k shared by
+// `n_v_heads / n_qk_heads` consecutive value heads, g the decay itself (not its log).
+//
+// The step is a pure HBM stream: 2*dk*dv*4 bytes of state traffic per head against
+// O(dk*dv) flops. The kernel reads every state element exactly once and writes it exactly
+// once. Both reductions over dk are taken on the *old* state while it sits in registers:
+//
+//   a = S0^T k,  c = S0^T q,  kq = k.q
+//   delta = beta*(v - g*a)
+//   o     = dk^-1/2 * (g*c + kq*delta)
+//   S1    = g*S0 + k delta^T
+//
+// which is the same update with the read-out folded in, so no second pass over S is needed.
+//
+// Work decomposition: a workgroup of 256 lanes (4 wavefronts) owns COLS consecutive value
+// columns of one head, all DK rows. Lane t holds the float4 column group (t % (COLS/4)) of
+// rows (t / (COLS/4)) + m*ROWS_PER_PASS. A wavefront load instruction therefore covers
+// 64/(COLS/4) full row segments of COLS*4 contiguous bytes: with COLS = 128 that is two
+// complete 512-byte state rows per instruction, 16 bytes per lane. Column sums are reduced
+// across the lanes of a wavefront with lane permutes and across the 4 wavefronts through
+// 4 KB of LDS. q, k are staged in LDS as fp32.
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <stdint.h>
+
+#include "launch_status.hpp"
+
+namespace {
+
+constexpr int DK = 128;
+constexpr int DV = 128;
+constexpr int THREADS = 256;
+constexpr int WAVES = THREADS / 64;
+
+__device__ __forceinline__ float to_f32(float x) { return x; }
+__device__ __forceinline__ float to_f32(__hip_bfloat16 x) { return __bfloat162float(x); }
+
+template <typename T, int COLS>
+__global__ __launch_bounds__(THREADS) void gdn_decode_kernel(
+    float* __restrict__ o, float* __restrict__ state, const T* __restrict__ q,
+    const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ g,
+    const float* __restrict__ beta, int n_v_heads, int n_qk_heads, float scale) {
+    constexpr int CG = COLS / 4;            // float4 column groups per row segment
+    constexpr int RPP = THREADS / CG;       // rows covered by one pass of the workgroup
+    constexpr int NP = DK / RPP;            // passes; float4 values held per lane
+    constexpr int ROWS_PER_WAVE = 64 / CG;  // rows of one pass that fall into one wavefront
+    constexpr int TILES = DV / COLS;        // workgroups per head
+
+    __shared__ float s_q[DK];
+    __shared__ float s_k[DK];
+    __shared__ float s_kq[WAVES];
+    __shared__ float4 s_red[2][WAVES][CG];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int cg = tid % CG;
+    const int r0 = tid / CG;
+
+    const int unit = blockIdx.x / TILES;  // b * n_v_heads + hv
+    const int tile = blockIdx.x % TILES;
+    const int b = unit / n_v_heads;
+    const int hv = unit % n_v_heads;
+    const int hq = hv / (n_v_heads / n_qk_heads);
+
+    float* S = state + (size_t)unit * (DK * DV) + tile * COLS + cg * 4;
+
+    // Issue the whole state tile's loads first; everything below overlaps their latency.
+    float4 s[NP];
+#pragma unroll
+    for (int m = 0; m < NP; ++m) {
+        s[m] = *reinterpret_cast<const float4*>(S + (size_t)(r0 + m * RPP) * DV);
+    }
+
+    const T* qh = q + ((size_t)b * n_qk_heads + hq) * DK;
+    const T* kh = k + ((size_t)b * n_qk_heads + hq) * DK;
+    float kq_part = 0.f;
+    if (tid < DK) {
+        const float qv = to_f32(qh[tid]);
+        const float kv = to_f32(kh[tid]);
+        s_q[tid] = qv;
+        s_k[tid] = kv;
+        kq_part = qv * kv;
+    }
+    if (tid < DK) {  // waves 0 and 1 (DK == 128): wavefront sum of k_i*q_i
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) kq_part += __shfl_xor(kq_part, off);
+        if (lane == 0) s_kq[wave] = kq_part;
+    }
+    const float4 vj = [&] {
+        const T* vh = v + (size_t)unit * DV + tile * COLS + cg * 4;
+        return make_float4(to_f32(vh[0]), to_f32(vh[1]), to_f32(vh[2]), to_f32(vh[3]));
+    }();
+    const float gh = g[unit];
+    const float bh = beta[unit];
+    __syncthreads();
+
+    // a = S0^T k and c = S0^T q over this lane's rows
+    float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 c = make_float4(0.f, 0.f, 0.f, 0.f);
+    float kr[NP];
+#pragma unroll
+    for (int m = 0; m < NP; ++m) {
+        const int r = r0 + m * RPP;
+        kr[m] = s_k[r];
+        const float qr = s_q[r];
+        a.x += s[m].x * kr[m]; a.y += s[m].y * kr[m]; a.z += s[m].z * kr[m]; a.w += s[m].w * kr[m];
+        c.x += s[m].x * qr;    c.y += s[m].y * qr;    c.z += s[m].z * qr;    c.w += s[m].w * qr;
+    }
+    // across the rows that share a wavefront (lane bits >= log2(CG))
+#pragma unroll
+    for (int off = 32; off >= CG; off >>= 1) {
+        a.x += __shfl_xor(a.x, off); a.y += __shfl_xor(a.y, off);
+        a.z += __shfl_xor(a.z, off); a.w += __shfl_xor(a.w, off);
+        c.x += __shfl_xor(c.x, off); c.y += __shfl_xor(c.y, off);
+        c.z += __shfl_xor(c.z, off); c.w += __shfl_xor(c.w, off);
+    }
+    if (lane < CG) {
+        s_red[0][wave][lane] = a;
+        s_red[1][wave][lane] = c;
+    }
+    __syncthreads();
+    a = s_red[0][0][cg];
+    c = s_red[1][0][cg];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) {
+        const float4 aw = s_red[0][w][cg];
+        const float4 cw = s_red[1][w][cg];
+        a.x += aw.x; a.y += aw.y; a.z += aw.z; a.w += aw.w;
+        c.x += cw.x; c.y += cw.y; c.z += cw.z; c.w += cw.w;
+    }
+    const float kq = s_kq[0] + s_kq[1];
+
+    float4 d;
+    d.x = bh * (vj.x - gh * a.x);
+    d.y = bh * (vj.y - gh * a.y);
+    d.z = bh * (vj.z - gh * a.z);
+    d.w = bh * (vj.w - gh * a.w);
+
+    if (r0 == 0) {
+        float4 ov;
+        ov.x = scale * (gh * c.x + kq * d.x);
+        ov.y = scale * (gh * c.y + kq * d.y);
+        ov.z = scale * (gh * c.z + kq * d.z);
+        ov.w = scale * (gh * c.w + kq * d.w);
+        *reinterpret_cast<float4*>(o + (size_t)unit * DV + tile * COLS + cg * 4) = ov;
+    }
+
+#pragma unroll
+    for (int m = 0; m < NP; ++m) {
+        float4 n;
+        n.x = gh * s[m].x + kr[m] * d.x;
+        n.y = gh * s[m].y + kr[m] * d.y;
+        n.z = gh * s[m].z + kr[m] * d.z;
+        n.w = gh * s[m].w + kr[m] * d.w;
+        *reinterpret_cast<float4*>(S + (size_t)(r0 + m * RPP) * DV) = n;
+    }
+}
+
+template <typename T>
+void launch(float* o, float* state, const void* q, const void* k, const void* v, const float* g,
+            const float* beta, int batch, int n_v_heads, int n_qk_heads, int config,
+            hipStream_t stream) {
+    const long units = (long)batch * n_v_heads;
+    const float scale = 0.08838834764831845f;  // 128^-1/2
+    const T* qt = static_cast<const T*>(q);
+    const T* kt = static_cast<const T*>(k);
+    const T* vt = static_cast<const T*>(v);
+    int cols = config == 1 ? 128 : config == 2 ? 64 : config == 3 ? 32 : 0;
+    if (cols == 0) cols = units >= 2048 ? 128 : 32;  // few heads: more, smaller workgroups
+    switch (cols) {
+        case 128:
+            gdn_decode_kernel<T, 128><<<dim3(units), THREADS, 0, stream>>>(
+                o, state, qt, kt, vt, g, beta, n_v_heads, n_qk_heads, scale);
+            break;
+        case 64:
+            gdn_decode_kernel<T, 64><<<dim3(units * 2), THREADS, 0, stream>>>(
+                o, state, qt, kt, vt, g, beta, n_v_heads, n_qk_heads, scale);
+            break;
+        default:
+            gdn_decode_kernel<T, 32><<<dim3(units * 4), THREADS, 0, stream>>>(
+                o, state, qt, kt, vt, g, beta, n_v_heads, n_qk_heads, scale);
+            break;
+    }
+}
+
+}  // namespace
+
+// o      [batch, n_v_heads, 128] fp32, written
+// state  [batch, n_v_heads, 128, 128] fp32, updated in place
+// q, k   [batch, n_qk_heads, 128]; v [batch, n_v_heads, 128]; all three fp32 (qkv_dtype 0)
+//        or bf16 (qkv_dtype 1)
+// g, beta [batch, n_v_heads] fp32
+// config: 0 picks the column tiling from the number of heads; 1, 2, 3 force workgroups of
+//         128, 64, 32 value columns.
+extern "C" void gdn_decode_launcher(float* o, float* state, const void* q, const void* k,
+                                    const void* v, const float* g, const float* beta, int batch,
+                                    int n_v_heads, int n_qk_heads, int dk, int dv, int qkv_dtype,
+                                    int config, hipStream_t stream) {
+    if (batch <= 0 || n_v_heads <= 0) return;
+    if (dk != DK || dv != DV || n_qk_heads <= 0 || n_v_heads % n_qk_heads != 0 ||
+        (qkv_dtype != 0 && qkv_dtype != 1) || (long)batch * n_v_heads * 4 > 0x7fffffffL) {
+        caa::set_status(CAA_UNSUPPORTED_SHAPE);
+        return;
+    }
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(o) | reinterpret_cast<uintptr_t>(state);
+    if (!o || !state || !q || !k || !v || !g || !beta || (bits & 15u) != 0) {
+        caa::set_status(CAA_BAD_ARGUMENT);
+        return;
+    }
+    if (qkv_dtype == 0) {
+        launch<float>(o, state, q, k, v, g, beta, batch, n_v_heads, n_qk_heads, config, stream);
+    } else {
+        launch<__hip_bfloat16>(o, state, q, k, v, g, beta, batch, n_v_heads, n_qk_heads, config,
+                               stream);
+    }
+}

@@ -1,0 +1,116 @@
+#!/usr/bin/env python3
+"""Differential check of ``ModelNew`` (the HIP extension) against the eager ``Model``.
+
+Behaviour follows the reference workspace's checker (agent_workdir/utils/verification.py:22-99):
+five rounds, each with inputs drawn afresh by ``get_inputs()``, both models on the GPU with
+``ModelNew`` loading ``Model``'s ``state_dict``, ``ModelNew.forward`` run with every public
+``torch.nn.functional`` callable replaced by a function that raises, outputs compared with
+``torch.testing.assert_close(atol=1e-2, rtol=1e-2)`` after a Python-type check, and the same
+``[PASS]`` lines. Any mismatch ends the process with an uncaught exception.
+
+Run from the workspace directory: ``python3 -m utils.verification``.
+"""
+
+from contextlib import contextmanager
+
+import torch
+import torch.nn.functional as F
+
+from model import Model, get_inputs, get_init_inputs
+from model_new import ModelNew
+
+NUM_CHECKS = 5
+ATOL = 1e-2
+RTOL = 1e-2
+
+
+def transform_tensors(tensors, fn):
+    """Apply ``fn`` to every tensor in a nest of lists/tuples/dicts (tuples become lists)."""
+    if isinstance(tensors, torch.Tensor):
+        return fn(tensors)
+    if isinstance(tensors, (list, tuple)):
+        return [transform_tensors(item, fn) for item in tensors]
+    if isinstance(tensors, dict):
+        return {key: transform_tensors(item, fn) for key, item in tensors.items()}
+    return tensors
+
+
+def check_equal(actual, expected):
+    assert type(actual) == type(expected), f"{type(actual)=} != {type(expected)=}"
+    if isinstance(actual, torch.Tensor):
+        torch.testing.assert_close(actual, expected, atol=ATOL, rtol=RTOL)
+    elif isinstance(actual, (list, tuple)):
+        assert len(actual) == len(expected), f"{len(actual)=} != {len(expected)=}"
+        for got, want in zip(actual, expected):
+            check_equal(got, want)
+    elif isinstance(actual, dict):
+        for key, want in expected.items():
+            assert key in actual, f"Missing key in output: {key}"
+            check_equal(actual[key], want)
+    elif isinstance(actual, (str, float, int)):
+        assert actual == expected, f"{actual=} != {expected=}"
+    else:
+        raise TypeError(f"Unsupported output type: {type(actual)}")
+
+
+def _make_blocker(name):
+    def blocked(*args, **kwargs):
+        raise RuntimeError(f"Function torch.nn.functional.{name} is not allowed in this context.")
+    return blocked
+
+
+@contextmanager
+def block_torch_functional(excludes=None):
+    """Inside the block every public callable of ``torch.nn.functional`` raises RuntimeError."""
+    excludes = set() if excludes is None else set(excludes)
+    saved = {}
+    for name in dir(F):
+        if name.startswith("_") or name in excludes:
+            continue
+        attr = getattr(F, name)
+        if callable(attr):
+            saved[name] = attr
+            setattr(F, name, _make_blocker(name))
+    try:
+        yield
+    finally:
+        for name, attr in saved.items():
+            setattr(F, name, attr)
+
+
+def _as_list(value):
+    return list(value) if isinstance(value, (list, tuple)) else [value]
+
+
+def initialize_models():
+    init_inputs = _as_list(get_init_inputs())
+    torch_model = Model(*init_inputs).eval().cuda()
+    cuda_model = ModelNew(*init_inputs).eval().cuda()
+    cuda_model.load_state_dict(torch_model.state_dict())
+    return torch_model, cuda_model
+
+
+def build_inputs():
+    torch_inputs = transform_tensors(_as_list(get_inputs()), lambda t: t.cuda())
+    cuda_inputs = transform_tensors(torch_inputs, lambda t: t.clone())
+    return torch_inputs, cuda_inputs
+
+
+def main():
+    torch_model, cuda_model = initialize_models()
+
+    with torch.no_grad():
+        for i in range(NUM_CHECKS):
+            torch_inputs, cuda_inputs = build_inputs()
+            torch_output = torch_model(*torch_inputs)
+            with block_torch_functional():
+                cuda_output = cuda_model(*cuda_inputs)
+            check_equal(cuda_output, torch_output)
+            print(f"[PASS] check {i + 1}/{NUM_CHECKS}")
+
+    torch.cuda.synchronize()
+    print("[PASS] verify success")
+
+
+if __name__ == "__main__":
+    main()

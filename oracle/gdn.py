@@ -1,0 +1,95 @@
+"""Oracle for the Gated DeltaNet single-token decode step (test infrastructure only).
+
+Specification restated (workload configs 0 and 1): per request b and value head h, with S the
+fp32 ``[dk, dv]`` state, ``g`` the decay itself and q/k shared by ``Hv // Hqk`` consecutive
+value heads (head ``h`` reads q/k head ``h // (Hv // Hqk)``)::
+
+    S = g*S;  S += beta * k (v - S^T k)^T;  o = S^T q * dk**-0.5
+
+The reference repository has no implementation of this operator; its model contract
+(``Model.forward`` / ``get_inputs`` / ``get_init_inputs``, agent_workdir/model.py:9-26) is
+what the functions below are shaped after.
+
+Pinned by (tests/test_oracle_gdn.py):
+  * ``gdn_decode_loops_f64``: float64 scalar loops written straight from the recurrence;
+  * invariants: beta=0 gives pure decay; g=1, beta=1, |k|=1 gives ``S'^T k == v``;
+    the folded single-pass identity ``o = scale*(g*S0^T q + (k.q)*delta)``;
+    GQA equals the ungrouped rule fed the repeated q/k heads;
+  * a golden fixture written from an independent third-party implementation of the same
+    recurrence (tests/golden/make_gdn_golden.py).
+"""
+
+import math
+
+import numpy as np
+import torch
+
+
+def gdn_decode_step(q, k, v, g, beta, state):
+    """Vectorised fp32 eager step. Mutates ``state`` in place and returns ``(o, state)``.
+
+    q, k: [B, Hqk, dk]; v: [B, Hv, dv]; g, beta: [B, Hv]; state: [B, Hv, dk, dv] fp32.
+    q/k/v may be bf16 or fp32; the arithmetic is fp32.
+    """
+    B, Hv, dk, dv = state.shape
+    rep = Hv // q.shape[1]
+    qf = q.float().repeat_interleave(rep, dim=1)
+    kf = k.float().repeat_interleave(rep, dim=1)
+    vf = v.float()
+    state.mul_(g.float()[:, :, None, None])
+    u = torch.einsum('bhij,bhi->bhj', state, kf)
+    delta = beta.float()[:, :, None] * (vf - u)
+    state.add_(kf[:, :, :, None] * delta[:, :, None, :])
+    o = torch.einsum('bhij,bhi->bhj', state, qf) * (dk ** -0.5)
+    return o, state
+
+
+def gdn_decode_loops_f64(q, k, v, g, beta, state):
+    """Scalar float64 loops over numpy arrays; returns ``(o, new_state)``, inputs untouched."""
+    q, k, v, g, beta, state = (np.asarray(x, dtype=np.float64) for x in (q, k, v, g, beta, state))
+    B, Hv, dk, dv = state.shape
+    rep = Hv // q.shape[1]
+    S = state.copy()
+    o = np.zeros((B, Hv, dv))
+    for b in range(B):
+        for h in range(Hv):
+            hq = h // rep
+            for i in range(dk):
+                for j in range(dv):
+                    S[b, h, i, j] *= g[b, h]
+            u = [sum(S[b, h, i, j] * k[b, hq, i] for i in range(dk)) for j in range(dv)]
+            for j in range(dv):
+                d = beta[b, h] * (v[b, h, j] - u[j])
+                for i in range(dk):
+                    S[b, h, i, j] += k[b, hq, i] * d
+            for j in range(dv):
+                o[b, h, j] = sum(S[b, h, i, j] * q[b, hq, i] for i in range(dk)) / math.sqrt(dk)
+    return o, S
+
+
+def gdn_make_inputs(batch, n_v_heads, n_qk_heads, dk=128, dv=128, qkv_dtype=torch.float32,
+                    generator=None):
+    """Synthetic inputs of the workload: q, k, v ~ N(0,1) with q and k L2-normalised per head in
+    fp32 before the cast to ``qkv_dtype``; g = exp(-0.5*softplus(N(0,1))); beta = sigmoid(N(0,1));
+    state ~ N(0, 0.02) fp32. Returns ``[q, k, v, g, beta, state]`` on the CPU."""
+    gen = generator
+    q = torch.randn(batch, n_qk_heads, dk, generator=gen)
+    k = torch.randn(batch, n_qk_heads, dk, generator=gen)
+    v = torch.randn(batch, n_v_heads, dv, generator=gen)
+    q = q / q.norm(dim=-1, keepdim=True)
+    k = k / k.norm(dim=-1, keepdim=True)
+    g = torch.exp(-0.5 * torch.nn.functional.softplus(torch.randn(batch, n_v_heads, generator=gen)))
+    beta = torch.sigmoid(torch.randn(batch, n_v_heads, generator=gen))
+    state = 0.02 * torch.randn(batch, n_v_heads, dk, dv, generator=gen)
+    return [q.to(qkv_dtype), k.to(qkv_dtype), v.to(qkv_dtype), g, beta, state]
+
+
+def gdn_close(actual, expected, rtol=1e-3):
+    """The fp32 tolerance of this operator: |a-b| <= rtol*|b| + rtol*rms(b).
+
+    A pure relative bound is ill-posed because outputs cross zero; the absolute floor is the
+    same fraction of the tensor's RMS."""
+    a = actual.double()
+    e = expected.double()
+    atol = rtol * e.pow(2).mean().sqrt()
+    return bool(((a - e).abs() <= rtol * e.abs() + atol).all())

@@ -1,0 +1,147 @@
+"""GPU parity of the GDN decode kernel against the oracle, through the C ABI.
+
+Tolerance (fp32 arithmetic): |a-b| <= 1e-3*|b| + 1e-3*rms(b) for output and state
+(oracle.gdn.gdn_close)."""
+import os
+import subprocess
+import sys
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import gdn
+
+pytestmark = pytest.mark.gpu
+REPO = Path(__file__).resolve().parent.parent
+GOLDEN = Path(__file__).parent / 'golden' / 'gdn_decode_golden.npz'
+
+
+def run_kernel(capi, dev, ins, config=0):
+    q, k, v, g, beta, state = (t.to(dev) for t in ins)
+    o = torch.full((state.shape[0], state.shape[1], state.shape[3]), float('nan'), device=dev)
+    capi.gdn_decode_launch(o, state, q, k, v, g, beta, config=config)
+    torch.cuda.synchronize()
+    return o.cpu(), state.cpu()
+
+
+@pytest.mark.parametrize('config', [0, 1, 2, 3])
+@pytest.mark.parametrize('shape', [(1, 16, 16, torch.float32), (3, 8, 4, torch.bfloat16),
+                                   (2, 6, 6, torch.bfloat16), (5, 4, 1, torch.float32)])
+def test_matches_oracle(capi, dev, shape, config):
+    B, Hv, Hqk, dt = shape
+    gen = torch.Generator().manual_seed(100 + B)
+    ins = gdn.gdn_make_inputs(B, Hv, Hqk, qkv_dtype=dt, generator=gen)
+    want_o, want_s = gdn.gdn_decode_step(*ins[:5], ins[5].clone())
+    o, s = run_kernel(capi, dev, ins, config)
+    assert gdn.gdn_close(o, want_o) and gdn.gdn_close(s, want_s)
+
+
+def test_workload_config0_fixed_seed(capi, dev):
+    gen = torch.Generator().manual_seed(20250)
+    ins = gdn.gdn_make_inputs(1, 16, 16, generator=gen)
+    want_o, want_s = gdn.gdn_decode_step(*ins[:5], ins[5].clone())
+    o, s = run_kernel(capi, dev, ins)
+    assert gdn.gdn_close(o, want_o) and gdn.gdn_close(s, want_s)
+    # and the reference harness's own bound
+    torch.testing.assert_close(o, want_o, atol=1e-2, rtol=1e-2)
+
+
+def test_golden_fixture(capi, dev):
+    z = np.load(GOLDEN)
+    ins = [torch.from_numpy(z[n]) for n in ('q', 'k', 'v', 'g', 'beta', 'state')]
+    o, s = run_kernel(capi, dev, ins)
+    assert gdn.gdn_close(o, torch.from_numpy(z['o']))
+    assert gdn.gdn_close(s, torch.from_numpy(z['new_state']))
+
+
+def test_several_steps_track_the_oracle(capi, dev):
+    gen = torch.Generator().manual_seed(5)
+    q, k, v, g, beta, state = gdn.gdn_make_inputs(2, 8, 4, qkv_dtype=torch.bfloat16, generator=gen)
+    ref_state = state.clone()
+    d_state = state.to(dev)
+    o = torch.empty(2, 8, 128, device=dev)
+    for step in range(6):
+        q, k, v, g, beta, _ = gdn.gdn_make_inputs(2, 8, 4, qkv_dtype=torch.bfloat16, generator=gen)
+        want_o, ref_state = gdn.gdn_decode_step(q, k, v, g, beta, ref_state)
+        capi.gdn_decode_launch(o, d_state, *(t.to(dev) for t in (q, k, v, g, beta)))
+        assert gdn.gdn_close(o.cpu(), want_o), step
+    assert gdn.gdn_close(d_state.cpu(), ref_state)
+
+
+def test_full_batched_workload_properties(capi, dev):
+    """Config 1 at full size (B=256, 32/16 heads, 537 MB of state), checked through properties
+    that need no CPU pass over the state: a sampled set of heads against the oracle, pure decay
+    for beta = 0 and the delta-rule write for g = beta = 1."""
+    B, Hv, Hqk = 256, 32, 16
+    gen = torch.Generator(device=dev).manual_seed(20251)
+    q = torch.randn(B, Hqk, 128, device=dev, generator=gen)
+    k = torch.randn(B, Hqk, 128, device=dev, generator=gen)
+    q = (q / q.norm(dim=-1, keepdim=True)).bfloat16()
+    k = (k / k.norm(dim=-1, keepdim=True)).bfloat16()
+    v = torch.randn(B, Hv, 128, device=dev, generator=gen).bfloat16()
+    g = torch.exp(-0.5 * torch.log1p(torch.exp(torch.randn(B, Hv, device=dev, generator=gen))))
+    beta = torch.sigmoid(torch.randn(B, Hv, device=dev, generator=gen))
+    state = 0.02 * torch.randn(B, Hv, 128, 128, device=dev, generator=gen)
+    o = torch.empty(B, Hv, 128, device=dev)
+
+    picks = [(0, 0), (0, 31), (17, 5), (128, 16), (255, 30), (255, 31)]
+    before = {p: state[p].cpu().clone() for p in picks}
+    capi.gdn_decode_launch(o, state, q, k, v, g, beta)
+    torch.cuda.synchronize()
+    for (b, h) in picks:
+        hq = h // 2
+        want_o, want_s = gdn.gdn_decode_step(
+            q[b, hq][None, None].cpu(), k[b, hq][None, None].cpu(), v[b, h][None, None].cpu(),
+            g[b, h][None, None].cpu(), beta[b, h][None, None].cpu(), before[(b, h)][None, None])
+        assert gdn.gdn_close(o[b, h].cpu()[None, None], want_o), (b, h)
+        assert gdn.gdn_close(state[b, h].cpu()[None, None], want_s), (b, h)
+
+    # beta = 0: the state is only scaled by g (bit-exact: one fp32 multiply per element)
+    snap = state.clone()
+    capi.gdn_decode_launch(o, state, q, k, v, g, torch.zeros_like(beta))
+    torch.cuda.synchronize()
+    assert torch.equal(state, snap * g[:, :, None, None])
+
+    # g = beta = 1: probing the new state with k gives S0^T k + |k|^2 (v - S0^T k), which is v
+    # up to the bf16 rounding of |k| = 1
+    kf = k.float().repeat_interleave(2, 1)
+    kn = (kf * kf).sum(-1, keepdim=True)
+    probe0 = torch.einsum('bhij,bhi->bhj', state, kf)
+    capi.gdn_decode_launch(o, state, q, k, v, torch.ones_like(g), torch.ones_like(beta))
+    torch.cuda.synchronize()
+    probe = torch.einsum('bhij,bhi->bhj', state, kf)
+    torch.testing.assert_close(probe, probe0 + kn * (v.float() - probe0), rtol=1e-4, atol=1e-4)
+    assert (probe - v.float()).abs().max().item() < 0.1
+
+
+@pytest.mark.parametrize('ws_config', ['0', '1'])
+def test_workspace_verification_flow(ws_config):
+    """`python3 -m utils.verification` from inside the workspace, as its user runs it."""
+    ws = REPO / 'cuda-agent_amd' / 'workspaces' / 'gdn_decode'
+    assert (ws / 'cuda_extension.so').exists(), 'workspace extension not built'
+    env = dict(os.environ, GDN_CONFIG=ws_config)
+    out = subprocess.run([sys.executable, '-m', 'utils.verification'], cwd=ws, env=env,
+                         capture_output=True, text=True, timeout=600)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert '[PASS] check 5/5' in out.stdout and '[PASS] verify success' in out.stdout
+
+
+def test_workspace_rejects_bad_inputs(dev):
+    ws = REPO / 'cuda-agent_amd' / 'workspaces' / 'gdn_decode'
+    code = (
+        "import torch, cuda_extension as e\n"
+        "d='cuda:0'\n"
+        "q=torch.zeros(1,2,128,device=d);v=torch.zeros(1,2,128,device=d);g=torch.ones(1,2,device=d)\n"
+        "s=torch.zeros(1,2,128,128,device=d)\n"
+        "o,s2=e.gdn_decode_forward(q,q,v,g,g,s,0); assert s2.data_ptr()==s.data_ptr() and o.shape==(1,2,128)\n"
+        "for bad in [lambda: e.gdn_decode_forward(q.cpu(),q,v,g,g,s,0),\n"
+        "            lambda: e.gdn_decode_forward(q.half(),q.half(),v.half(),g,g,s,0),\n"
+        "            lambda: e.gdn_decode_forward(q,q,v,g,g,s[:,:,:64].contiguous(),0),\n"
+        "            lambda: e.gdn_decode_forward(q,q,v,g,g,s.transpose(2,3),0)]:\n"
+        "    try: bad(); raise SystemExit('accepted a bad input')\n"
+        "    except RuntimeError: pass\n"
+        "print('ok')\n")
+    out = subprocess.run([sys.executable, '-c', code], cwd=ws, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0 and 'ok' in out.stdout, out.stdout + out.stderr

@@ -1,0 +1,106 @@
+"""Pins the GDN decode oracle: brute force, invariants and a third-party golden fixture."""
+from pathlib import Path
+
+import numpy as np
+import torch
+
+from oracle import gdn
+
+GOLDEN = Path(__file__).parent / 'golden' / 'gdn_decode_golden.npz'
+
+
+def _tiny(seed=0, B=2, Hv=4, Hqk=2, dk=8, dv=4):
+    gen = torch.Generator().manual_seed(seed)
+    return gdn.gdn_make_inputs(B, Hv, Hqk, dk, dv, generator=gen)
+
+
+def test_vectorised_step_matches_float64_loops():
+    q, k, v, g, beta, state = _tiny()
+    want_o, want_s = gdn.gdn_decode_loops_f64(*(t.numpy() for t in (q, k, v, g, beta, state)))
+    o, s = gdn.gdn_decode_step(q, k, v, g, beta, state.clone())
+    np.testing.assert_allclose(o.numpy(), want_o, rtol=1e-5, atol=1e-7)
+    np.testing.assert_allclose(s.numpy(), want_s, rtol=1e-5, atol=1e-7)
+
+
+def test_state_is_updated_in_place_and_returned():
+    q, k, v, g, beta, state = _tiny(1)
+    before = state.clone()
+    o, s = gdn.gdn_decode_step(q, k, v, g, beta, state)
+    assert s.data_ptr() == state.data_ptr()
+    assert not torch.equal(before, state)
+
+
+def test_beta_zero_is_pure_decay():
+    q, k, v, g, beta, state = _tiny(2)
+    s0 = state.clone()
+    o, s = gdn.gdn_decode_step(q, k, v, g, torch.zeros_like(beta), state)
+    torch.testing.assert_close(s, s0 * g[:, :, None, None])
+    rep = 2
+    want_o = torch.einsum('bhij,bhi->bhj', s0, q.repeat_interleave(rep, 1)) * g[:, :, None] * 8 ** -0.5
+    torch.testing.assert_close(o, want_o, rtol=1e-5, atol=1e-7)
+
+
+def test_delta_rule_writes_v_under_key():
+    # g = 1, beta = 1, |k| = 1: after the step the state returns v when probed with k.
+    q, k, v, g, beta, state = _tiny(3)
+    o, s = gdn.gdn_decode_step(q, k, v, torch.ones_like(g), torch.ones_like(beta), state)
+    probe = torch.einsum('bhij,bhi->bhj', s, k.repeat_interleave(2, 1))
+    torch.testing.assert_close(probe, v, rtol=1e-5, atol=1e-6)
+
+
+def test_folded_single_pass_identity():
+    # o = scale*(g*S0^T q + (k.q)*delta) with delta = beta*(v - g*S0^T k): the form the kernel uses
+    q, k, v, g, beta, state = _tiny(4, dk=16, dv=8)
+    s0 = state.double()
+    qd, kd = q.double().repeat_interleave(2, 1), k.double().repeat_interleave(2, 1)
+    a = torch.einsum('bhij,bhi->bhj', s0, kd)
+    c = torch.einsum('bhij,bhi->bhj', s0, qd)
+    gd, bd = g.double()[:, :, None], beta.double()[:, :, None]
+    delta = bd * (v.double() - gd * a)
+    want_o = 16 ** -0.5 * (gd * c + (kd * qd).sum(-1, keepdim=True) * delta)
+    want_s = gd[..., None] * s0 + kd[..., None] * delta[:, :, None, :]
+    o, s = gdn.gdn_decode_step(q, k, v, g, beta, state)
+    torch.testing.assert_close(o.double(), want_o, rtol=1e-5, atol=1e-7)
+    torch.testing.assert_close(s.double(), want_s, rtol=1e-5, atol=1e-7)
+
+
+def test_gqa_equals_repeated_heads():
+    q, k, v, g, beta, state = _tiny(5, Hv=6, Hqk=3)
+    o1, s1 = gdn.gdn_decode_step(q, k, v, g, beta, state.clone())
+    o2, s2 = gdn.gdn_decode_step(q.repeat_interleave(2, 1), k.repeat_interleave(2, 1), v, g, beta,
+                                 state.clone())
+    assert torch.equal(o1, o2) and torch.equal(s1, s2)
+
+
+def test_linear_in_state_and_v():
+    q, k, v, g, beta, state = _tiny(6)
+    o1, s1 = gdn.gdn_decode_step(q, k, v, g, beta, state.clone())
+    o2, s2 = gdn.gdn_decode_step(q, k, 3 * v, g, beta, 3 * state.clone())
+    torch.testing.assert_close(o2, 3 * o1, rtol=1e-5, atol=1e-7)
+    torch.testing.assert_close(s2, 3 * s1, rtol=1e-5, atol=1e-7)
+
+
+def test_bf16_inputs_are_upcast():
+    q, k, v, g, beta, state = _tiny(7)
+    qb, kb, vb = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    o1, _ = gdn.gdn_decode_step(qb, kb, vb, g, beta, state.clone())
+    o2, _ = gdn.gdn_decode_step(qb.float(), kb.float(), vb.float(), g, beta, state.clone())
+    assert o1.dtype == torch.float32 and torch.equal(o1, o2)
+
+
+def test_input_distribution():
+    gen = torch.Generator().manual_seed(11)
+    q, k, v, g, beta, state = gdn.gdn_make_inputs(8, 32, 16, generator=gen)
+    torch.testing.assert_close(q.norm(dim=-1), torch.ones(8, 16), rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(k.norm(dim=-1), torch.ones(8, 16), rtol=1e-5, atol=1e-5)
+    assert (g > 0).all() and (g <= 1).all() and (beta > 0).all() and (beta < 1).all()
+    assert abs(state.std().item() - 0.02) < 1e-3
+    assert q.shape == (8, 16, 128) and v.shape == (8, 32, 128) and state.shape == (8, 32, 128, 128)
+
+
+def test_golden_fixture_from_third_party_recurrence():
+    z = np.load(GOLDEN)
+    ins = [torch.from_numpy(z[n]) for n in ('q', 'k', 'v', 'g', 'beta', 'state')]
+    o, s = gdn.gdn_decode_step(*ins[:5], ins[5].clone())
+    np.testing.assert_allclose(o.numpy(), z['o'], rtol=2e-5, atol=1e-7)
+    np.testing.assert_allclose(s.numpy(), z['new_state'], rtol=2e-5, atol=1e-7)
