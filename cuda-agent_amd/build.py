@@ -19,6 +19,7 @@ WORKSPACES_DIR = PACKAGE_DIR / 'workspaces'
 
 GPU_ARCH = 'gfx950'
 DEVICE_FLAGS = [
+    '-Wno-inline-asm',
     '-O3', '-std=c++17', '-fPIC', f'--offload-arch={GPU_ARCH}', '-fno-gpu-rdc',
     '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
 ]

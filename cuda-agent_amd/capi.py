@@ -8,7 +8,7 @@ every output and scratch buffer is allocated by the caller, as the launcher ABI 
 """
 
 import ctypes
-from ctypes import c_float, c_int, c_void_p
+from ctypes import c_float, c_int, c_size_t, c_void_p
 
 from . import CAPI_LIBRARY
 
@@ -20,6 +20,10 @@ SIGNATURES = {
     'axpby_launcher': (None, [_P, _P, _P, c_float, c_int, c_int, _P]),
     'gdn_decode_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int,
                                    c_int, c_int, _P]),
+    'sparse_mla_decode_launcher': (None, [_P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int,
+                                          c_int, c_int, c_float, c_int, c_int, _P]),
+    'sparse_mla_decode_num_splits': (c_int, [c_int, c_int, c_int, c_int]),
+    'sparse_mla_decode_workspace_bytes': (c_size_t, [c_int, c_int, c_int, c_int]),
 }
 
 STATUS_NAMES = {0: 'ok', 1: 'unsupported shape', 2: 'bad argument', 3: 'workspace too small'}
@@ -105,3 +109,30 @@ def gdn_decode_launch(o, state, q, k, v, g, beta, config=0, stream=None):
                                   0 if q.dtype == torch.float32 else 1, config, _stream(stream))
     check_status('gdn_decode_launcher')
     return o, state
+
+
+def sparse_mla_workspace_bytes(batch, n_heads, topk, config=0):
+    return int(library().sparse_mla_decode_workspace_bytes(batch, n_heads, topk, config))
+
+
+def sparse_mla_decode_launch(out, q, kv, idx, workspace, sm_scale=192 ** -0.5, config=0, stream=None):
+    """out [B,H,512] (bf16, or fp32 for the unrounded values) <- attention of q [B,H,576] over rows idx [B,topk] of kv [B,N,576].
+    ``workspace`` is a uint8 device tensor of at least ``sparse_mla_workspace_bytes`` bytes."""
+    import torch
+    _device_contiguous(out=out, q=q, kv=kv, idx=idx, workspace=workspace)
+    B, H, d_qk = q.shape
+    N = kv.shape[1]
+    topk = idx.shape[1]
+    d_v = out.shape[2]
+    _require(q.dtype == kv.dtype == torch.bfloat16, 'sparse_mla: q, kv must be bf16')
+    _require(out.dtype in (torch.bfloat16, torch.float32), 'sparse_mla: out must be bf16 or fp32')
+    _require(idx.dtype == torch.int32, 'sparse_mla: idx must be int32')
+    _require(tuple(kv.shape) == (B, N, d_qk) and tuple(idx.shape) == (B, topk), 'sparse_mla: kv/idx shape')
+    _require(tuple(out.shape) == (B, H, d_v), 'sparse_mla: out shape')
+    library().sparse_mla_decode_launcher(_ptr(out), _ptr(q), _ptr(kv), _ptr(idx), _ptr(workspace),
+                                         workspace.numel() * workspace.element_size(), B, H, N, topk,
+                                         d_qk, d_v, float(sm_scale),
+                                         0 if out.dtype == torch.bfloat16 else 1, config,
+                                         _stream(stream))
+    check_status('sparse_mla_decode_launcher')
+    return out

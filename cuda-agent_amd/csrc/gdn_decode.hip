@@ -33,17 +33,36 @@ namespace {
 
 constexpr int DK = 128;
 constexpr int DV = 128;
-constexpr int THREADS = 256;
-constexpr int WAVES = THREADS / 64;
 
 __device__ __forceinline__ float to_f32(float x) { return x; }
 __device__ __forceinline__ float to_f32(__hip_bfloat16 x) { return __bfloat162float(x); }
 
-template <typename T, int COLS>
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// NT marks the access as streaming (no reuse expected), one 16-byte instruction either way.
+__device__ __forceinline__ float4 load_state(const float* p, bool nt) {
+    if (nt) {
+        const floatx4 r = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(p));
+        return make_float4(r.x, r.y, r.z, r.w);
+    }
+    return *reinterpret_cast<const float4*>(p);
+}
+
+__device__ __forceinline__ void store_state(float* p, float4 x, bool nt) {
+    if (nt) {
+        floatx4 r = {x.x, x.y, x.z, x.w};
+        __builtin_nontemporal_store(r, reinterpret_cast<floatx4*>(p));
+    } else {
+        *reinterpret_cast<float4*>(p) = x;
+    }
+}
+
+template <typename T, int COLS, int THREADS, int NT>
 __global__ __launch_bounds__(THREADS) void gdn_decode_kernel(
     float* __restrict__ o, float* __restrict__ state, const T* __restrict__ q,
     const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ g,
     const float* __restrict__ beta, int n_v_heads, int n_qk_heads, float scale) {
+    constexpr int WAVES = THREADS / 64;
     constexpr int CG = COLS / 4;            // float4 column groups per row segment
     constexpr int RPP = THREADS / CG;       // rows covered by one pass of the workgroup
     constexpr int NP = DK / RPP;            // passes; float4 values held per lane
@@ -73,7 +92,7 @@ __global__ __launch_bounds__(THREADS) void gdn_decode_kernel(
     float4 s[NP];
 #pragma unroll
     for (int m = 0; m < NP; ++m) {
-        s[m] = *reinterpret_cast<const float4*>(S + (size_t)(r0 + m * RPP) * DV);
+        s[m] = load_state(S + (size_t)(r0 + m * RPP) * DV, NT == 1 || NT == 2);
     }
 
     const T* qh = q + ((size_t)b * n_qk_heads + hq) * DK;
@@ -157,35 +176,48 @@ __global__ __launch_bounds__(THREADS) void gdn_decode_kernel(
         n.y = gh * s[m].y + kr[m] * d.y;
         n.z = gh * s[m].z + kr[m] * d.z;
         n.w = gh * s[m].w + kr[m] * d.w;
-        *reinterpret_cast<float4*>(S + (size_t)(r0 + m * RPP) * DV) = n;
+        store_state(S + (size_t)(r0 + m * RPP) * DV, n, NT == 1 || NT == 3);
     }
+}
+
+template <typename T, int COLS, int THREADS, int NT>
+void launch_variant(float* o, float* state, const T* q, const T* k, const T* v, const float* g,
+                    const float* beta, int units, int n_v_heads, int n_qk_heads,
+                    hipStream_t stream) {
+    const float scale = 0.08838834764831845f;  // 128^-1/2
+    gdn_decode_kernel<T, COLS, THREADS, NT><<<dim3(units * (DV / COLS)), THREADS, 0, stream>>>(
+        o, state, q, k, v, g, beta, n_v_heads, n_qk_heads, scale);
 }
 
 template <typename T>
 void launch(float* o, float* state, const void* q, const void* k, const void* v, const float* g,
             const float* beta, int batch, int n_v_heads, int n_qk_heads, int config,
             hipStream_t stream) {
-    const long units = (long)batch * n_v_heads;
-    const float scale = 0.08838834764831845f;  // 128^-1/2
+    const int units = batch * n_v_heads;
     const T* qt = static_cast<const T*>(q);
     const T* kt = static_cast<const T*>(k);
     const T* vt = static_cast<const T*>(v);
-    int cols = config == 1 ? 128 : config == 2 ? 64 : config == 3 ? 32 : 0;
-    if (cols == 0) cols = units >= 2048 ? 128 : 32;  // few heads: more, smaller workgroups
-    switch (cols) {
-        case 128:
-            gdn_decode_kernel<T, 128><<<dim3(units), THREADS, 0, stream>>>(
-                o, state, qt, kt, vt, g, beta, n_v_heads, n_qk_heads, scale);
-            break;
-        case 64:
-            gdn_decode_kernel<T, 64><<<dim3(units * 2), THREADS, 0, stream>>>(
-                o, state, qt, kt, vt, g, beta, n_v_heads, n_qk_heads, scale);
-            break;
-        default:
-            gdn_decode_kernel<T, 32><<<dim3(units * 4), THREADS, 0, stream>>>(
-                o, state, qt, kt, vt, g, beta, n_v_heads, n_qk_heads, scale);
-            break;
+    if (config <= 0 || config > 12) config = units >= 2048 ? 9 : 12;  // few heads: smaller tiles
+#define GDN_VARIANT(id, cols, threads, nt)                                                     \
+    case id:                                                                                   \
+        launch_variant<T, cols, threads, nt>(o, state, qt, kt, vt, g, beta, units, n_v_heads,  \
+                                             n_qk_heads, stream);                              \
+        break;
+    switch (config) {
+        GDN_VARIANT(1, 128, 256, 0)
+        GDN_VARIANT(2, 64, 256, 0)
+        GDN_VARIANT(3, 32, 256, 0)
+        GDN_VARIANT(4, 128, 512, 0)
+        GDN_VARIANT(5, 128, 256, 1)
+        GDN_VARIANT(6, 128, 512, 1)
+        GDN_VARIANT(7, 64, 512, 0)
+        GDN_VARIANT(8, 128, 1024, 0)
+        GDN_VARIANT(9, 128, 1024, 1)
+        GDN_VARIANT(10, 128, 1024, 2)
+        GDN_VARIANT(11, 128, 1024, 3)
+        GDN_VARIANT(12, 32, 256, 1)
     }
+#undef GDN_VARIANT
 }
 
 }  // namespace

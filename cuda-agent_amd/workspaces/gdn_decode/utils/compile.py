@@ -28,6 +28,7 @@ GPU_ARCH = 'gfx950'
 HOST_FLAGS = ['-O3', '-std=c++17', '-fPIC']
 # Packed-FP32 instruction selection is switched off for every device translation unit.
 DEVICE_FLAGS = [
+    '-Wno-inline-asm',
     '-O3', '-std=c++17', '-fPIC', f'--offload-arch={GPU_ARCH}', '-fno-gpu-rdc',
     '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
 ]

@@ -68,6 +68,34 @@ void gdn_decode_launcher(float* o, float* state, const void* q, const void* k, c
                          int n_qk_heads, int dk, int dv, int qkv_dtype, int config,
                          hipStream_t stream);
 
+/* Sparse-MLA decode attention (workload config 3 of the benchmark definition; launcher
+ * pattern agent_workdir/kernels/axpby.cu:12-20). Per request every head attends to the rows
+ * of that request's latent cache listed in idx:
+ *   out[b,h,:] = softmax_k(q[b,h,:] . kv[b,idx[b,k],:] * sm_scale) @ kv[b,idx[b,k],:512]
+ *   out  [batch, n_heads, 512], written: bf16 if out_dtype == 0 (the operator's output), fp32
+ *        if out_dtype == 1 (the same values before the final rounding; lets a checker separate
+ *        arithmetic error from the bf16 output rounding)
+ *   q    [batch, n_heads, 576] bf16
+ *   kv   [batch, n_kv_rows, 576] bf16
+ *   idx  [batch, topk] int32; entries < 0 or >= n_kv_rows are padding and are skipped
+ *   workspace: device scratch of sparse_mla_decode_workspace_bytes(...) bytes (partial
+ *              outputs of the key splits), allocated by the caller
+ * Supported: d_qk == 576, d_v == 512, n_heads in {32, 64} or a multiple of 128. All pointers
+ * 16-byte aligned.
+ * config: 0 chooses the number of key splits so that about one workgroup per CU is resident;
+ * n > 0 forces n splits (raised if a split would exceed 2048 rows, lowered to the number of
+ * 32-row tiles). */
+void sparse_mla_decode_launcher(void* out, const void* q, const void* kv, const int* idx,
+                                void* workspace, size_t workspace_bytes, int batch, int n_heads,
+                                int n_kv_rows, int topk, int d_qk, int d_v, float sm_scale,
+                                int out_dtype, int config, hipStream_t stream);
+
+/* Number of key splits the launcher will use for these sizes and this config. */
+int sparse_mla_decode_num_splits(int batch, int n_heads, int topk, int config);
+
+/* Bytes of workspace sparse_mla_decode_launcher needs for these sizes and this config. */
+size_t sparse_mla_decode_workspace_bytes(int batch, int n_heads, int topk, int config);
+
 #ifdef __cplusplus
 }
 #endif

@@ -52,13 +52,16 @@ def test_ctypes_table_matches_header():
                 assert ctype is ctypes.c_void_p, (name, arg)
             elif arg.startswith('float'):
                 assert ctype is ctypes.c_float, (name, arg)
+            elif arg.startswith('size_t'):
+                assert ctype is ctypes.c_size_t, (name, arg)
             elif arg.startswith('int'):
                 assert ctype is ctypes.c_int, (name, arg)
 
 
 def test_library_has_no_torch_dependency():
     from cuda_agent_amd import CAPI_LIBRARY
-    needed = subprocess.run(['readelf', '-d', str(CAPI_LIBRARY)], capture_output=True, text=True).stdout
+    out = subprocess.run(['readelf', '-d', str(CAPI_LIBRARY)], capture_output=True, text=True).stdout
+    needed = ' '.join(line for line in out.splitlines() if 'NEEDED' in line)
     assert 'libamdhip64' in needed
     assert 'torch' not in needed and 'c10' not in needed and 'python' not in needed
 
