@@ -56,19 +56,25 @@ __device__ __forceinline__ int swizzled_slot(int row, int chunk) {
     return row * ROW_CHUNKS + ((chunk & ~7) | ((chunk ^ row) & 7));
 }
 
-// One wavefront's share of a tile load: LDS slots [first_slot, first_slot + 64*N) in lane order.
+// One wavefront's share of a tile: with NW wavefronts each owns 32/NW consecutive rows, fetched by
+// PER_WAVE global->LDS instructions of 64 lanes x 16 bytes.
 template <int NW>
-__device__ __forceinline__ void issue_tile_load(uint4* tile, const char* kv_b, const int* s_idx_tile,
-                                                bool has_padding, int wave, int lane) {
-    constexpr int PER_WAVE = TILE_CHUNKS / 64 / NW;  // 36 wave-instructions per tile
-    // The slot -> (row, chunk) arithmetic is a handful of integer operations per load. Hiding the
-    // lane number from the optimiser here keeps it from precomputing all of them before the
-    // tile loop and holding (or spilling) two registers per load for the whole kernel.
-    asm volatile("" : "+v"(lane));
-#pragma unroll
-    for (int i = 0; i < PER_WAVE; ++i) {
+struct TileLoader {
+    static constexpr int PER_WAVE = TILE_CHUNKS / 64 / NW;  // 36 / NW
+    const char* kv_b;
+    int wave;
+    int lane;
+
+    // Instruction i of this wavefront's share of `tile`.
+    __device__ __forceinline__ void issue(uint4* tile, const int* s_idx_tile, bool has_padding,
+                                          int i) const {
+        // Hiding the lane number from the optimiser keeps the slot -> (row, chunk) arithmetic
+        // (a handful of integer operations) from being precomputed for all loads before the
+        // tile loop, which would hold two registers per load for the whole kernel.
+        int l = lane;
+        asm volatile("" : "+v"(l));
         const int inst = wave * PER_WAVE + i;
-        const int slot = inst * 64 + lane;
+        const int slot = inst * 64 + l;
         const int row = slot / ROW_CHUNKS;
         const int pos = slot - row * ROW_CHUNKS;
         const int chunk = (pos & ~7) | ((pos ^ row) & 7);
@@ -91,12 +97,27 @@ __device__ __forceinline__ void issue_tile_load(uint4* tile, const char* kv_b, c
             tile[slot] = make_uint4(0u, 0u, 0u, 0u);
         }
     }
-}
+
+    __device__ __forceinline__ void issue_all(uint4* tile, const int* s_idx_tile,
+                                              bool has_padding) const {
+#pragma unroll
+        for (int i = 0; i < PER_WAVE; ++i) issue(tile, s_idx_tile, has_padding, i);
+    }
+};
 
 struct SoftmaxState {
-    float m;  // running max of the scaled scores (log2 domain); same in lanes l and l^32
+    float m;  // reference exponent of the accumulator (log2 domain); same in lanes l and l^32
     float l;  // running sum of exp2(s - m) over the rows this lane has seen
 };
+
+// The accumulator is kept relative to a per-head reference exponent m, which moves whenever a
+// score exceeds it by more than FRAME_SLACK powers of two. With slack 0 this is the usual strict
+// running maximum: the largest probability of a head is exactly 1, which is what keeps the
+// bf16 rounding of the probabilities below the 2e-2*rms bound on heads that one row dominates
+// (a slack of 8 measured 2.0e-2 on the full workload against 0.9e-2 for slack 0). The price is
+// the 256-register rescale of the accumulator on almost every tile, since some head out of a
+// wavefront's 32 nearly always sees a new maximum.
+constexpr float FRAME_SLACK = 0.f;
 
 // Per-lane byte offsets into a tile, computed once. With the XOR swizzle every LDS address of
 // the inner loops is one of these six values plus a compile-time constant, so the reads use
@@ -128,13 +149,17 @@ __device__ __forceinline__ LaneOffsets make_lane_offsets(int lane) {
 
 typedef const __attribute__((address_space(3))) char* lds_bytes;
 
-// Everything a wavefront does with one resident tile. LDS reads run one group of four MFMAs
-// ahead of their use; the scheduling fences keep the compiler from hoisting all 36 + 64 reads
-// to the top (which would need more registers than the 112 left beside Q and the accumulator).
+// Everything a wavefront does with one resident tile. `prefetch(i)` issues instruction i of the
+// wavefront's share of a later tile; the calls are spread over the QK^T loop so that the
+// address arithmetic overlaps the matrix pipeline and the memory system sees a steady stream.
+// LDS reads run two groups ahead of the MFMAs that consume them; the scheduling fences keep the
+// compiler from hoisting all 36 + 64 reads to the top (which would need more registers than
+// the ~110 left beside Q and the accumulator).
+template <int PREFETCH_COUNT, typename Prefetch>
 __device__ __forceinline__ void process_tile(const uint4* tile, const int* s_idx_tile, bool masked,
                                              const bf16x8 (&qreg)[K_STEPS], floatx16 (&acc)[DV_TILES],
                                              SoftmaxState& st, const LaneOffsets& off,
-                                             float scale_log2, int lane) {
+                                             float scale_log2, int lane, Prefetch prefetch) {
     typedef const __attribute__((address_space(3))) uintx4* lds_x4;
     typedef shortx4 __attribute__((address_space(3)))* lds_s4;
     const int half = lane >> 5;
@@ -145,43 +170,36 @@ __device__ __forceinline__ void process_tile(const uint4* tile, const int* s_idx
 
     // S^T[row, head] = sum_d K[row, d] Q[head, d]
     floatx16 s = {0};
-    asm volatile("" : "+v"(s));  // keep S out of the accumulation registers, which O^T fills
+    asm volatile("" : "+v"(s));  // keep S out of the accumulation registers
     {
-        constexpr int G = 2;
+        constexpr int G = 2;                 // MFMAs per group
         constexpr int GROUPS = K_STEPS / G;  // 18
-        uintx4 kbuf[2][G];
-#pragma unroll
-        for (int j = 0; j < G; ++j) kbuf[0][j] = *(lds_x4)(base + off.qk[j & 3] + (j >> 2) * 128);
-#pragma unroll
-        for (int g = 0; g < GROUPS; ++g) {
-            if (g + 1 < GROUPS) {
-#pragma unroll
-                for (int j = 0; j < G; ++j) {
-                    const int ks = G * (g + 1) + j;
-                    kbuf[(g + 1) & 1][j] = *(lds_x4)(base + off.qk[ks & 3] + (ks >> 2) * 128);
-                }
-            }
+        constexpr int DEPTH = 2;             // groups of LDS reads in flight
+        uintx4 kbuf[DEPTH][G];
+        auto k_read = [&](int g) {
 #pragma unroll
             for (int j = 0; j < G; ++j) {
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kbuf[g & 1][j]),
-                                                            qreg[G * g + j], s, 0, 0, 0);
+                const int ks = G * g + j;
+                kbuf[g % DEPTH][j] = *(lds_x4)(base + off.qk[ks & 3] + (ks >> 2) * 128);
+            }
+        };
+#pragma unroll
+        for (int g = 0; g < DEPTH - 1; ++g) k_read(g);
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g) {
+            if (g + DEPTH - 1 < GROUPS) k_read(g + DEPTH - 1);
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kbuf[g % DEPTH][0]),
+                                                        qreg[G * g], s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kbuf[g % DEPTH][1]),
+                                                        qreg[G * g + 1], s, 0, 0, 0);
+#pragma unroll
+            for (int i = g * PREFETCH_COUNT / GROUPS; i < (g + 1) * PREFETCH_COUNT / GROUPS; ++i) {
+                prefetch(i);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
     }
-
-    constexpr int PV_STEPS = 2 * DV_TILES;  // (k-step, dv tile) pairs, 32 MFMAs
-    constexpr int PV_GROUP = 4;
-    shortx4 vbuf[2][PV_GROUP][2];
-    auto pv_read = [&](int step, shortx4 (&dst)[2]) {
-        const int ks = step / DV_TILES;
-        const int t = step % DV_TILES;
-#pragma unroll
-        for (int rr = 0; rr < 2; ++rr) {
-            dst[rr] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (lds_s4)(base + off.pv[t & 1] + (16 * ks + 8 * rr) * ROW_BYTES + (t >> 1) * 128));
-        }
-    };
+    asm volatile("" : "+v"(s));  // the softmax arithmetic below wants S in ordinary VGPRs
 
     // register i of `s` is row 8*(i/4) + 4*half + i%4 of the tile, head = lane % 32
     float tmax = -INFINITY;
@@ -197,23 +215,31 @@ __device__ __forceinline__ void process_tile(const uint4* tile, const int* s_idx
 #pragma unroll
     for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, s[i]);
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
-    const float m_new = fmaxf(st.m, tmax);
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;  // all rows masked so far
-    const float alpha = __builtin_amdgcn_exp2f(st.m - m_use);
+
+    // Move the reference exponent only when this tile exceeds it by more than FRAME_SLACK (or
+    // when it is still unset). alpha rescales what has been accumulated so far.
+    const bool move = tmax > st.m + FRAME_SLACK || st.m == -INFINITY;
+    const float m_new = move ? tmax : st.m;
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;  // every row so far was padding
+    const float alpha = move ? __builtin_amdgcn_exp2f(st.m - m_use) : 1.f;
+    const bool rescale = move && st.l != 0.f;  // nothing accumulated yet: nothing to rescale
     st.m = m_new;
 
     float psum = 0.f;
     bf16x8 p[2];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-        const float e = __builtin_amdgcn_exp2f(s[i] - m_use);
-        psum += e;
-        p[i / 8][i % 8] = (__bf16)e;
+        const __bf16 e = (__bf16)__builtin_amdgcn_exp2f(s[i] - m_use);
+        p[i / 8][i % 8] = e;
+        // The normaliser sums the probabilities as rounded, i.e. exactly the weights the PV
+        // product uses: the output is then a true convex combination of rows, and where one row
+        // dominates a head the rounding error of its weight cancels between numerator and
+        // denominator.
+        psum += (float)e;
     }
     st.l = st.l * alpha + psum;
 
-    // rescale the accumulator only when some head's maximum moved
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+    if (__builtin_amdgcn_ballot_w64(rescale) != 0) {
 #pragma unroll
         for (int t = 0; t < DV_TILES; ++t) {
             // The empty asm statements pin the tile to accumulation registers on both sides
@@ -229,6 +255,18 @@ __device__ __forceinline__ void process_tile(const uint4* tile, const int* s_idx
 
     // O^T[dv, head] += V^T[dv, row] P^T[row, head]; k index 8*half + 4*rr + e of k-step ks is
     // tile row 16*ks + 8*rr + 4*half + e for both operands.
+    constexpr int PV_STEPS = 2 * DV_TILES;  // (k-step, dv tile) pairs, 32 MFMAs
+    constexpr int PV_GROUP = 4;
+    shortx4 vbuf[2][PV_GROUP][2];
+    auto pv_read = [&](int step, shortx4 (&dst)[2]) {
+        const int ks = step / DV_TILES;
+        const int t = step % DV_TILES;
+#pragma unroll
+        for (int rr = 0; rr < 2; ++rr) {
+            dst[rr] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (lds_s4)(base + off.pv[t & 1] + (16 * ks + 8 * rr) * ROW_BYTES + (t >> 1) * 128));
+        }
+    };
 #pragma unroll
     for (int j = 0; j < PV_GROUP; ++j) pv_read(j, vbuf[0][j]);
 #pragma unroll
@@ -264,7 +302,7 @@ __global__ __launch_bounds__(64 * NW) void sparse_mla_split_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ kv, const int* __restrict__ idx,
     float* __restrict__ o_part, float* __restrict__ lse_part, int n_heads, int n_kv_rows, int topk,
     int rows_per_split, float scale_log2) {
-    constexpr int PER_WAVE = TILE_CHUNKS / 64 / NW;
+    constexpr int PER_WAVE = TileLoader<NW>::PER_WAVE;
     // Three separately named tile buffers: the compiler then knows which in-flight
     // global->LDS loads an LDS read can depend on and does not drain all of them.
     __shared__ uint4 tile0[TILE_CHUNKS];
@@ -304,12 +342,12 @@ __global__ __launch_bounds__(64 * NW) void sparse_mla_split_kernel(
     __syncthreads();
     const int first_masked_tile = s_first_masked_tile;
 
-    const char* kv_b = reinterpret_cast<const char*>(kv) + (size_t)b * n_kv_rows * ROW_BYTES;
+    const TileLoader<NW> loader{
+        reinterpret_cast<const char*>(kv) + (size_t)b * n_kv_rows * ROW_BYTES, wave, lane};
 
     // prologue: tiles 0 and 1 in flight
-    if (n_tiles > 0) issue_tile_load<NW>(tile0, kv_b, s_idx, 0 >= first_masked_tile, wave, lane);
-    if (n_tiles > 1)
-        issue_tile_load<NW>(tile1, kv_b, s_idx + TILE_ROWS, 1 >= first_masked_tile, wave, lane);
+    if (n_tiles > 0) loader.issue_all(tile0, s_idx, 0 >= first_masked_tile);
+    if (n_tiles > 1) loader.issue_all(tile1, s_idx + TILE_ROWS, 1 >= first_masked_tile);
 
     // Q^T operand: lane holds Q[head0 + lane%32][16*ks + 8*(lane/32) .. +7]
     bf16x8 qreg[K_STEPS];
@@ -320,7 +358,6 @@ __global__ __launch_bounds__(64 * NW) void sparse_mla_split_kernel(
             qreg[ks] = *reinterpret_cast<const bf16x8*>(qrow + 16 * ks);
         }
     }
-
     // Make the Q loads complete here, once (the empty asm statements are uses of the loaded
     // registers): a wait for them inside the tile loop would also wait, on every pass, for
     // the tile loads issued behind them.
@@ -336,8 +373,8 @@ __global__ __launch_bounds__(64 * NW) void sparse_mla_split_kernel(
     // Three-stage ring. At the top of step t the loads of tiles t and t+1 are outstanding;
     // waiting until at most one tile's worth of loads is in flight therefore completes tile t.
     // (A tile with padding rows issues an unknown number of loads, so next to such a tile the
-    // wait is for everything.) Tile t+2 is issued after the barrier, into the buffer every
-    // wavefront finished reading in step t-1.
+    // wait is for everything.) Tile t+2 is issued during step t, after the barrier, into the
+    // buffer every wavefront finished reading in step t-1.
 #define MLA_STEP(CUR, NXT2, T)                                                                  \
     {                                                                                           \
         if ((T) + 1 < n_tiles && (T) + 1 < first_masked_tile)                                   \
@@ -346,11 +383,13 @@ __global__ __launch_bounds__(64 * NW) void sparse_mla_split_kernel(
             wait_vmcnt<0>();                                                                    \
         __builtin_amdgcn_s_barrier();                                                           \
         asm volatile("" ::: "memory");                                                          \
-        if ((T) + 2 < n_tiles)                                                                  \
-            issue_tile_load<NW>(NXT2, kv_b, s_idx + ((T) + 2) * TILE_ROWS,                      \
-                                (T) + 2 >= first_masked_tile, wave, lane);                      \
-        process_tile(CUR, s_idx + (T) * TILE_ROWS, (T) >= first_masked_tile, qreg, acc, st, off,  \
-                     scale_log2, lane);                                                         \
+        const bool more = (T) + 2 < n_tiles;                                                    \
+        const bool pad2 = (T) + 2 >= first_masked_tile;                                         \
+        const int* idx2 = s_idx + ((T) + 2) * TILE_ROWS;                                        \
+        process_tile<PER_WAVE>(CUR, s_idx + (T) * TILE_ROWS, (T) >= first_masked_tile, qreg, acc, \
+                               st, off, scale_log2, lane, [&](int i) {                          \
+                                   if (more) loader.issue(NXT2, idx2, pad2, i);                 \
+                               });                                                              \
     }
     for (int t = 0; t < n_tiles; t += 3) {
         MLA_STEP(tile0, tile2, t)
@@ -359,24 +398,41 @@ __global__ __launch_bounds__(64 * NW) void sparse_mla_split_kernel(
     }
 #undef MLA_STEP
 
-    // epilogue: normalise, write partial output [b, split, head, dv] and log2-sum-exp
+    // Epilogue: normalise and write the partial output [b, split, head, dv] and the
+    // log2-sum-exp. The accumulator is O^T (a lane holds 4 consecutive dv of one head, lanes
+    // run over heads), so it goes through LDS, 128 dv at a time in a region private to the
+    // wavefront, to leave as 512-byte row segments.
     const float l_total = st.l + __shfl_xor(st.l, 32);
     const float inv_l = l_total > 0.f ? 1.f / l_total : 0.f;
-    const int head = head0 + (lane & 31);
     const int half = lane >> 5;
-    const size_t part = ((size_t)b * n_splits + split) * n_heads + head;
-    float* o_row = o_part + part * D_V;
-#pragma unroll
-    for (int t = 0; t < DV_TILES; ++t) {
-#pragma unroll
-        for (int qd = 0; qd < 4; ++qd) {
-            floatx4 v = {acc[t][4 * qd] * inv_l, acc[t][4 * qd + 1] * inv_l,
-                         acc[t][4 * qd + 2] * inv_l, acc[t][4 * qd + 3] * inv_l};
-            *reinterpret_cast<floatx4*>(o_row + 32 * t + 8 * qd + 4 * half) = v;
-        }
-    }
+    const size_t part0 = ((size_t)b * n_splits + split) * n_heads + head0;
     if (half == 0) {
-        lse_part[part] = l_total > 0.f ? st.m + __builtin_amdgcn_logf(l_total) : -INFINITY;
+        // v_log_f32 is a base-2 logarithm
+        lse_part[part0 + lane] = l_total > 0.f ? st.m + __builtin_amdgcn_logf(l_total) : -INFINITY;
+    }
+    __syncthreads();  // every wavefront is done with the tile buffers
+    constexpr int STAGE_STRIDE = 128 + 4;  // floats per staged head row (padded against conflicts)
+    float* stage = reinterpret_cast<float*>(wave < 2 ? tile0 : tile1) + (wave & 1) * (32 * STAGE_STRIDE);
+    float* o_rows = o_part + part0 * D_V;
+#pragma unroll
+    for (int ps = 0; ps < 4; ++ps) {
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) {
+            const floatx16 a = acc[4 * ps + tt];
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd) {
+                floatx4 v = {a[4 * qd] * inv_l, a[4 * qd + 1] * inv_l, a[4 * qd + 2] * inv_l,
+                             a[4 * qd + 3] * inv_l};
+                *reinterpret_cast<floatx4*>(stage + (lane & 31) * STAGE_STRIDE + 32 * tt + 8 * qd +
+                                            4 * half) = v;
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < 16; ++it) {
+            const int r = 2 * it + half;
+            const floatx4 v = *reinterpret_cast<const floatx4*>(stage + r * STAGE_STRIDE + 4 * (lane & 31));
+            *reinterpret_cast<floatx4*>(o_rows + (size_t)r * D_V + 128 * ps + 4 * (lane & 31)) = v;
+        }
     }
 }
 
