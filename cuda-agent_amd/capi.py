@@ -24,6 +24,17 @@ SIGNATURES = {
                                           c_int, c_int, c_float, c_int, c_int, _P]),
     'sparse_mla_decode_num_splits': (c_int, [c_int, c_int, c_int, c_int]),
     'sparse_mla_decode_workspace_bytes': (c_size_t, [c_int, c_int, c_int, c_int]),
+    'moe_route_launcher': (None, [_P, _P, _P, c_int, c_int, c_int, c_int, _P]),
+    'moe_sort_launcher': (None, [_P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P]),
+    'moe_quant_bf16_launcher': (None, [_P, _P, _P, c_int, c_int, c_int, _P]),
+    'moe_gate_up_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int,
+                                    c_int, _P]),
+    'moe_down_launcher': (None, [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P]),
+    'moe_combine_launcher': (None, [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P]),
+    'moe_fp8_workspace_bytes': (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
+    'moe_fp8_workspace_layout': (None, [_P, c_int, c_int, c_int, c_int, c_int]),
+    'moe_fp8_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int,
+                                c_int, c_int, c_int, _P]),
 }
 
 STATUS_NAMES = {0: 'ok', 1: 'unsupported shape', 2: 'bad argument', 3: 'workspace too small'}
@@ -135,4 +146,102 @@ def sparse_mla_decode_launch(out, q, kv, idx, workspace, sm_scale=192 ** -0.5, c
                                          0 if out.dtype == torch.bfloat16 else 1, config,
                                          _stream(stream))
     check_status('sparse_mla_decode_launcher')
+    return out
+
+
+MOE_WORKSPACE_FIELDS = ('ids', 'weights', 'expert_offsets', 'sorted_pairs', 'pair_pos', 'x_q', 'x_s',
+                        'h_q', 'h_s', 'y')
+
+
+def moe_workspace_bytes(tokens, hidden, inter, n_experts, top_k=8):
+    return int(library().moe_fp8_workspace_bytes(tokens, hidden, inter, n_experts, top_k))
+
+
+def moe_workspace_views(workspace, tokens, hidden, inter, n_experts, top_k=8):
+    """Typed views of the intermediate buffers inside a workspace tensor (uint8, 1-D)."""
+    import torch
+    offs = (c_size_t * 10)()
+    library().moe_fp8_workspace_layout(offs, tokens, hidden, inter, n_experts, top_k)
+    pairs = tokens * top_k
+    spec = {
+        'ids': (torch.int32, (tokens, top_k)), 'weights': (torch.float32, (tokens, top_k)),
+        'expert_offsets': (torch.int32, (n_experts + 1,)), 'sorted_pairs': (torch.int32, (pairs,)),
+        'pair_pos': (torch.int32, (pairs,)), 'x_q': (torch.float8_e4m3fn, (tokens, hidden)),
+        'x_s': (torch.float32, (tokens, hidden // 128)), 'h_q': (torch.float8_e4m3fn, (pairs, inter)),
+        'h_s': (torch.float32, (pairs, inter // 128)), 'y': (torch.float32, (pairs, hidden)),
+    }
+    views = {}
+    for name, off in zip(MOE_WORKSPACE_FIELDS, offs):
+        dtype, shape = spec[name]
+        n = 1
+        for d in shape:
+            n *= d
+        nbytes = n * torch.empty((), dtype=dtype).element_size()
+        views[name] = workspace[off:off + nbytes].view(dtype).view(shape)
+    return views
+
+
+def moe_route_launch(ids, weights, logits, stream=None):
+    import torch
+    _device_contiguous(ids=ids, weights=weights, logits=logits)
+    T, E = logits.shape
+    k = ids.shape[1]
+    _require(logits.dtype == torch.float32 and weights.dtype == torch.float32 and ids.dtype == torch.int32,
+             'moe_route: dtypes')
+    _require(tuple(ids.shape) == (T, k) and tuple(weights.shape) == (T, k), 'moe_route: shapes')
+    library().moe_route_launcher(_ptr(ids), _ptr(weights), _ptr(logits), T, E, k, 0, _stream(stream))
+    check_status('moe_route_launcher')
+    return ids, weights
+
+
+def moe_sort_launch(ids, n_experts, stream=None):
+    """Returns (sorted_pairs, pair_pos, expert_offsets) int32 device tensors."""
+    import torch
+    _device_contiguous(ids=ids)
+    _require(ids.dtype == torch.int32 and ids.dim() == 2, 'moe_sort: ids must be int32 [T, k]')
+    T, k = ids.shape
+    dev = ids.device
+    sorted_pairs = torch.empty(T * k, dtype=torch.int32, device=dev)
+    pair_pos = torch.empty(T * k, dtype=torch.int32, device=dev)
+    offsets = torch.empty(n_experts + 1, dtype=torch.int32, device=dev)
+    scratch = torch.empty(((T + 255) // 256) * n_experts, dtype=torch.int32, device=dev)
+    library().moe_sort_launcher(_ptr(sorted_pairs), _ptr(pair_pos), _ptr(offsets), _ptr(scratch),
+                                _ptr(ids), T, n_experts, k, 0, _stream(stream))
+    check_status('moe_sort_launcher')
+    return sorted_pairs, pair_pos, offsets
+
+
+def moe_quant_bf16_launch(q, scales, x, stream=None):
+    import torch
+    _device_contiguous(q=q, scales=scales, x=x)
+    R, C = x.shape
+    _require(x.dtype == torch.bfloat16 and scales.dtype == torch.float32, 'moe_quant: dtypes')
+    _require(q.element_size() == 1 and tuple(q.shape) == (R, C), 'moe_quant: q must be 1-byte [R, C]')
+    _require(tuple(scales.shape) == (R, C // 128), 'moe_quant: scales shape')
+    library().moe_quant_bf16_launcher(_ptr(q), _ptr(scales), _ptr(x), R, C, 0, _stream(stream))
+    check_status('moe_quant_bf16_launcher')
+    return q, scales
+
+
+def moe_fp8_launch(out, x, logits, w13_q, w13_s, w2_q, w2_s, workspace, top_k=8, config=0, stream=None):
+    """The whole layer; ``out`` [T, H] bf16 (or fp32 for the unrounded values)."""
+    import torch
+    _device_contiguous(out=out, x=x, logits=logits, w13_q=w13_q, w13_s=w13_s, w2_q=w2_q, w2_s=w2_s,
+                       workspace=workspace)
+    T, H = x.shape
+    E, I2, _ = w13_q.shape
+    I = I2 // 2
+    _require(x.dtype == torch.bfloat16 and logits.dtype == torch.float32, 'moe_fp8: x bf16, logits fp32')
+    _require(out.dtype in (torch.bfloat16, torch.float32) and tuple(out.shape) == (T, H), 'moe_fp8: out')
+    _require(w13_q.element_size() == 1 and w2_q.element_size() == 1, 'moe_fp8: weights must be e4m3')
+    _require(tuple(w13_q.shape) == (E, 2 * I, H) and tuple(w2_q.shape) == (E, H, I), 'moe_fp8: weight shapes')
+    _require(tuple(w13_s.shape) == (E, 2 * I // 128, H // 128) and tuple(w2_s.shape) == (E, H // 128, I // 128),
+             'moe_fp8: scale shapes')
+    _require(w13_s.dtype == torch.float32 and w2_s.dtype == torch.float32, 'moe_fp8: scales fp32')
+    _require(tuple(logits.shape) == (T, E), 'moe_fp8: logits shape')
+    library().moe_fp8_launcher(_ptr(out), _ptr(x), _ptr(logits), _ptr(w13_q), _ptr(w13_s), _ptr(w2_q),
+                               _ptr(w2_s), _ptr(workspace), workspace.numel() * workspace.element_size(),
+                               T, H, I, E, top_k, 0 if out.dtype == torch.bfloat16 else 1, config,
+                               _stream(stream))
+    check_status('moe_fp8_launcher')
     return out

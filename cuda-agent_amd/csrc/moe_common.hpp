@@ -1,0 +1,61 @@
+// Shared declarations of the FP8 block-scaled MoE kernels (route/sort, quantise, grouped GEMMs,
+// combine). Each stage has its own extern "C" launcher; moe_fp8_launcher chains them.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace moe {
+
+constexpr int GROUP = 128;            // quantisation group along K, and weight block edge
+constexpr float E4M3_MAX = 448.f;
+constexpr float AMAX_FLOOR = 1e-12f;  // scale of an all-zero group: 1e-12 / 448
+constexpr int SORT_CHUNK_TOKENS = 256;
+
+// Device scratch of one forward pass, carved from the caller's workspace.
+struct Workspace {
+    int* ids;             // [T*k]  expert of every (token, slot) pair, slots by descending logit
+    float* weights;       // [T*k]  routing weight of the pair
+    int* chunk_hist;      // [chunks*E] pairs of each expert in each 256-token chunk, then their
+                          //           exclusive prefix over chunks
+    int* expert_offsets;  // [E+1]  first sorted position of every expert
+    int* sorted_pairs;    // [T*k]  flat pair index at each sorted position
+    int* pair_pos;        // [T*k]  sorted position of each flat pair index
+    uint8_t* x_q;         // [T*H]  e4m3 activations
+    float* x_s;           // [T*H/128]
+    uint8_t* h_q;         // [T*k*I] e4m3 silu(g)*u, rows in sorted order
+    float* h_s;           // [T*k*I/128]
+    float* y;             // [T*k*H] expert outputs, rows in sorted order
+    size_t bytes;
+};
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+inline Workspace carve_workspace(void* base, int tokens, int hidden, int inter, int n_experts,
+                                 int top_k) {
+    Workspace w{};
+    size_t off = 0;
+    char* p = static_cast<char*>(base);
+    auto take = [&](size_t bytes) {
+        char* r = p ? p + off : nullptr;
+        off += align_up(bytes, 256);
+        return r;
+    };
+    const size_t pairs = (size_t)tokens * top_k;
+    const size_t chunks = (tokens + SORT_CHUNK_TOKENS - 1) / SORT_CHUNK_TOKENS;
+    w.ids = reinterpret_cast<int*>(take(pairs * 4));
+    w.weights = reinterpret_cast<float*>(take(pairs * 4));
+    w.chunk_hist = reinterpret_cast<int*>(take(chunks * n_experts * 4));
+    w.expert_offsets = reinterpret_cast<int*>(take(((size_t)n_experts + 1) * 4));
+    w.sorted_pairs = reinterpret_cast<int*>(take(pairs * 4));
+    w.pair_pos = reinterpret_cast<int*>(take(pairs * 4));
+    w.x_q = reinterpret_cast<uint8_t*>(take((size_t)tokens * hidden));
+    w.x_s = reinterpret_cast<float*>(take((size_t)tokens * (hidden / GROUP) * 4));
+    w.h_q = reinterpret_cast<uint8_t*>(take(pairs * inter));
+    w.h_s = reinterpret_cast<float*>(take(pairs * (inter / GROUP) * 4));
+    w.y = reinterpret_cast<float*>(take(pairs * hidden * 4));
+    w.bytes = off;
+    return w;
+}
+
+}  // namespace moe

@@ -1,0 +1,135 @@
+// Weighted combine of the expert outputs, and the launcher that runs the whole FP8 MoE layer:
+//   route -> sort -> quantise x -> gate/up GEMM (+SiLU*mul, requantise) -> down GEMM -> combine.
+#include <hip/hip_bf16.h>
+
+#include "launch_status.hpp"
+#include "moe_common.hpp"
+
+extern "C" void moe_route_launcher(int* ids, float* weights, const float* logits, int tokens,
+                                   int n_experts, int top_k, int config, hipStream_t stream);
+extern "C" void moe_sort_launcher(int* sorted_pairs, int* pair_pos, int* expert_offsets,
+                                  int* chunk_scratch, const int* ids, int tokens, int n_experts,
+                                  int top_k, int config, hipStream_t stream);
+extern "C" void moe_quant_bf16_launcher(void* q, float* scales, const void* x, int rows, int cols,
+                                        int config, hipStream_t stream);
+extern "C" void moe_gate_up_launcher(void* h_q, float* h_s, const void* x_q, const float* x_s,
+                                     const void* w13_q, const float* w13_s, const int* sorted_pairs,
+                                     const int* expert_offsets, int tokens, int hidden, int inter,
+                                     int n_experts, int top_k, int config, hipStream_t stream);
+extern "C" void moe_down_launcher(float* y, const void* h_q, const float* h_s, const void* w2_q,
+                                  const float* w2_s, const int* expert_offsets, int tokens, int hidden,
+                                  int inter, int n_experts, int top_k, int config, hipStream_t stream);
+
+namespace {
+
+using namespace moe;
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+
+// out[t, :] = sum_k weights[t, k] * y[pair_pos[t*top_k + k], :], k ascending, fp32.
+// One workgroup per token, 4 columns per lane and pass.
+template <typename OUT>
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y,
+                                                          const float* __restrict__ weights,
+                                                          const int* __restrict__ pair_pos,
+                                                          OUT* __restrict__ out, int hidden,
+                                                          int top_k) {
+    const int t = blockIdx.x;
+    for (int c = threadIdx.x * 4; c < hidden; c += 1024) {
+        floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+        for (int k = 0; k < top_k; ++k) {
+            const int pos = pair_pos[(size_t)t * top_k + k];
+            const float w = weights[(size_t)t * top_k + k];
+            const floatx4 v = *reinterpret_cast<const floatx4*>(y + (size_t)pos * hidden + c);
+            acc += v * w;
+        }
+        OUT* dst = out + (size_t)t * hidden + c;
+        if constexpr (sizeof(OUT) == 4) {
+            *reinterpret_cast<floatx4*>(dst) = acc;
+        } else {
+            bf16x4 r = {(__bf16)acc.x, (__bf16)acc.y, (__bf16)acc.z, (__bf16)acc.w};
+            *reinterpret_cast<bf16x4*>(dst) = r;
+        }
+    }
+}
+
+}  // namespace
+
+// out [tokens, hidden] (bf16 if out_dtype == 0, fp32 if 1) from y [tokens*top_k, hidden] fp32 in
+// sorted order, weights [tokens, top_k], pair_pos [tokens*top_k].
+extern "C" void moe_combine_launcher(void* out, const float* y, const float* weights,
+                                     const int* pair_pos, int tokens, int hidden, int top_k,
+                                     int out_dtype, int config, hipStream_t stream) {
+    (void)config;
+    if (tokens <= 0) return;
+    if (hidden <= 0 || hidden % 4 != 0 || top_k <= 0 || (out_dtype != 0 && out_dtype != 1)) {
+        caa::set_status(CAA_UNSUPPORTED_SHAPE);
+        return;
+    }
+    if (!out || !y || !weights || !pair_pos || (reinterpret_cast<uintptr_t>(y) & 15u) ||
+        (reinterpret_cast<uintptr_t>(out) & 15u)) {
+        caa::set_status(CAA_BAD_ARGUMENT);
+        return;
+    }
+    if (out_dtype == 0) {
+        moe_combine_kernel<__bf16><<<tokens, 256, 0, stream>>>(y, weights, pair_pos,
+                                                              static_cast<__bf16*>(out), hidden, top_k);
+    } else {
+        moe_combine_kernel<float><<<tokens, 256, 0, stream>>>(y, weights, pair_pos,
+                                                             static_cast<float*>(out), hidden, top_k);
+    }
+}
+
+extern "C" size_t moe_fp8_workspace_bytes(int tokens, int hidden, int inter, int n_experts,
+                                          int top_k) {
+    if (tokens <= 0 || hidden <= 0 || inter <= 0 || n_experts <= 0 || top_k <= 0) return 0;
+    return moe::carve_workspace(nullptr, tokens, hidden, inter, n_experts, top_k).bytes;
+}
+
+// Byte offsets of the intermediate buffers inside the workspace, in the order
+// ids, weights, expert_offsets, sorted_pairs, pair_pos, x_q, x_s, h_q, h_s, y
+// (for checkers that compare the stages against a reference).
+extern "C" void moe_fp8_workspace_layout(size_t* offsets10, int tokens, int hidden, int inter,
+                                         int n_experts, int top_k) {
+    char* base = reinterpret_cast<char*>(uintptr_t{4096});
+    const moe::Workspace w = moe::carve_workspace(base, tokens, hidden, inter, n_experts, top_k);
+    const void* ptrs[10] = {w.ids, w.weights, w.expert_offsets, w.sorted_pairs, w.pair_pos,
+                            w.x_q, w.x_s,     w.h_q,            w.h_s,          w.y};
+    for (int i = 0; i < 10; ++i) offsets10[i] = static_cast<const char*>(ptrs[i]) - base;
+}
+
+// The whole layer. out [tokens, hidden] bf16 (out_dtype 0) or fp32 (out_dtype 1).
+// config: 0 = defaults; 1, 2, 4 force 16, 32, 64 pairs per pass of the grouped GEMMs.
+extern "C" void moe_fp8_launcher(void* out, const void* x, const float* logits, const void* w13_q,
+                                 const float* w13_s, const void* w2_q, const float* w2_s,
+                                 void* workspace, size_t workspace_bytes, int tokens, int hidden,
+                                 int inter, int n_experts, int top_k, int out_dtype, int config,
+                                 hipStream_t stream) {
+    if (tokens <= 0) return;
+    if (hidden <= 0 || inter <= 0 || hidden % GROUP != 0 || inter % GROUP != 0 || n_experts <= 0 ||
+        n_experts > 512 || top_k <= 0 || top_k > 64 || top_k > n_experts ||
+        (long)tokens * top_k > 0x7fffffffL / 4 || (out_dtype != 0 && out_dtype != 1)) {
+        caa::set_status(CAA_UNSUPPORTED_SHAPE);
+        return;
+    }
+    if (!out || !x || !logits || !w13_q || !w13_s || !w2_q || !w2_s || !workspace ||
+        (reinterpret_cast<uintptr_t>(workspace) & 255u)) {
+        caa::set_status(CAA_BAD_ARGUMENT);
+        return;
+    }
+    const moe::Workspace w = moe::carve_workspace(workspace, tokens, hidden, inter, n_experts, top_k);
+    if (workspace_bytes < w.bytes) {
+        caa::set_status(CAA_WORKSPACE_TOO_SMALL);
+        return;
+    }
+    moe_route_launcher(w.ids, w.weights, logits, tokens, n_experts, top_k, 0, stream);
+    moe_sort_launcher(w.sorted_pairs, w.pair_pos, w.expert_offsets, w.chunk_hist, w.ids, tokens,
+                      n_experts, top_k, 0, stream);
+    moe_quant_bf16_launcher(w.x_q, w.x_s, x, tokens, hidden, 0, stream);
+    moe_gate_up_launcher(w.h_q, w.h_s, w.x_q, w.x_s, w13_q, w13_s, w.sorted_pairs, w.expert_offsets,
+                         tokens, hidden, inter, n_experts, top_k, config, stream);
+    moe_down_launcher(w.y, w.h_q, w.h_s, w2_q, w2_s, w.expert_offsets, tokens, hidden, inter,
+                      n_experts, top_k, config, stream);
+    moe_combine_launcher(out, w.y, w.weights, w.pair_pos, tokens, hidden, top_k, out_dtype, 0, stream);
+}

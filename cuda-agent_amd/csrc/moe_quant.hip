@@ -1,0 +1,56 @@
+// Activation quantisation: bf16 rows -> e4m3 codes with one fp32 scale per 128-wide group.
+//   scale = max(amax, 1e-12) / 448;  code = e4m3_rne(clamp(v / scale, -448, 448))
+// One wavefront per (row, group), two elements per lane. The division is IEEE fp32 so that the
+// codes are bit-identical to a CPU evaluation of the same formula; v_cvt_pk_fp8_f32 rounds to
+// nearest even but does not saturate (465 -> NaN), hence the clamp.
+#include <hip/hip_bf16.h>
+
+#include "launch_status.hpp"
+#include "moe_common.hpp"
+
+namespace {
+
+using namespace moe;
+
+__global__ __launch_bounds__(256) void moe_quant_bf16_kernel(const __hip_bfloat16* __restrict__ x,
+                                                             uint8_t* __restrict__ q,
+                                                             float* __restrict__ scales,
+                                                             long n_groups) {
+    const int lane = threadIdx.x & 63;
+    const long g = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (g >= n_groups) return;
+    const unsigned raw = *reinterpret_cast<const unsigned*>(x + g * GROUP + 2 * lane);
+    const float v0 = __uint_as_float(raw << 16);
+    const float v1 = __uint_as_float(raw & 0xffff0000u);
+    float amax = fmaxf(fabsf(v0), fabsf(v1));
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
+    const float scale = fmaxf(amax, AMAX_FLOOR) / E4M3_MAX;
+    const float a = fminf(fmaxf(v0 / scale, -E4M3_MAX), E4M3_MAX);
+    const float b = fminf(fmaxf(v1 / scale, -E4M3_MAX), E4M3_MAX);
+    const int packed = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+    *reinterpret_cast<uint16_t*>(q + g * GROUP + 2 * lane) = (uint16_t)(packed & 0xffff);
+    if (lane == 0) scales[g] = scale;
+}
+
+}  // namespace
+
+// q [rows, cols] e4m3 codes and scales [rows, cols/128] fp32 from x [rows, cols] bf16.
+extern "C" void moe_quant_bf16_launcher(void* q, float* scales, const void* x, int rows, int cols,
+                                        int config, hipStream_t stream) {
+    (void)config;
+    if (rows <= 0 || cols <= 0) return;
+    if (cols % GROUP != 0) {
+        caa::set_status(CAA_UNSUPPORTED_SHAPE);
+        return;
+    }
+    if (!q || !scales || !x || (reinterpret_cast<uintptr_t>(x) & 3u) ||
+        (reinterpret_cast<uintptr_t>(q) & 1u)) {
+        caa::set_status(CAA_BAD_ARGUMENT);
+        return;
+    }
+    const long n_groups = (long)rows * (cols / GROUP);
+    const long blocks = (n_groups + 3) / 4;
+    moe_quant_bf16_kernel<<<dim3((unsigned)blocks), 256, 0, stream>>>(
+        static_cast<const __hip_bfloat16*>(x), static_cast<uint8_t*>(q), scales, n_groups);
+}

@@ -1,0 +1,193 @@
+// MoE routing and the deterministic sort of (token, slot) pairs by expert.
+//
+// route:  one wavefront per token. The token's 8 experts are its 8 largest logits, ties going
+//         to the lower expert id, listed in that order; weight = sigmoid(logit) normalised over
+//         the 8. Ranking uses the logits themselves, which orders exactly as an exact sigmoid
+//         would and does not depend on how a sigmoid implementation rounds.
+// sort:   stable counting sort in three small kernels, all integer and order-independent:
+//         per-chunk histograms (256 tokens per chunk), an exclusive scan over chunks and
+//         experts, and a scatter in which lane e of a workgroup walks its chunk's pairs in
+//         flat order and hands out expert e's positions one by one.
+#include "launch_status.hpp"
+#include "moe_common.hpp"
+
+namespace {
+
+using namespace moe;
+
+__device__ __forceinline__ unsigned long long rank_key(float logit, int id) {
+    logit += 0.f;  // -0 -> +0, so that the two zeros tie
+    unsigned u = __float_as_uint(logit);
+    u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);  // monotone in the float order
+    return ((unsigned long long)u << 32) | (unsigned)(0x7fffffff - id);  // lower id wins a tie
+}
+
+template <int PER_LANE>
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits,
+                                                        int* __restrict__ ids,
+                                                        float* __restrict__ weights, int tokens,
+                                                        int n_experts, int top_k) {
+    const int lane = threadIdx.x & 63;
+    const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= tokens) return;
+    unsigned long long key[PER_LANE];
+#pragma unroll
+    for (int j = 0; j < PER_LANE; ++j) {
+        const int e = j * 64 + lane;
+        key[j] = e < n_experts ? rank_key(logits[(size_t)t * n_experts + e], e) : 0ull;
+    }
+    float my_score = 0.f;  // lane k keeps the k-th choice
+    int my_id = 0;
+    float total = 0.f;
+    for (int k = 0; k < top_k; ++k) {
+        unsigned long long best = 0ull;
+#pragma unroll
+        for (int j = 0; j < PER_LANE; ++j) best = key[j] > best ? key[j] : best;
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            const unsigned long long other = __shfl_xor(best, off);
+            best = other > best ? other : best;
+        }
+        const int id = 0x7fffffff - (int)(unsigned)(best & 0xffffffffull);
+#pragma unroll
+        for (int j = 0; j < PER_LANE; ++j) {
+            if (j * 64 + lane == id) key[j] = 0ull;  // taken
+        }
+        const float logit = logits[(size_t)t * n_experts + id];
+        const float score = 1.f / (1.f + expf(-logit));
+        total += score;
+        if (lane == k) {
+            my_score = score;
+            my_id = id;
+        }
+    }
+    if (lane < top_k) {
+        ids[(size_t)t * top_k + lane] = my_id;
+        weights[(size_t)t * top_k + lane] = my_score / total;
+    }
+}
+
+// chunk_hist[chunk][e] = number of pairs of chunk `chunk` routed to expert e
+__global__ __launch_bounds__(256) void moe_hist_kernel(const int* __restrict__ ids,
+                                                       int* __restrict__ chunk_hist, int pairs,
+                                                       int pairs_per_chunk, int n_experts) {
+    extern __shared__ int s_hist[];
+    for (int e = threadIdx.x; e < n_experts; e += 256) s_hist[e] = 0;
+    __syncthreads();
+    const int begin = blockIdx.x * pairs_per_chunk;
+    int end = begin + pairs_per_chunk;
+    if (end > pairs) end = pairs;
+    for (int p = begin + threadIdx.x; p < end; p += 256) atomicAdd(&s_hist[ids[p]], 1);
+    __syncthreads();
+    for (int e = threadIdx.x; e < n_experts; e += 256) {
+        chunk_hist[(size_t)blockIdx.x * n_experts + e] = s_hist[e];
+    }
+}
+
+// In place: chunk_hist[chunk][e] becomes the first sorted position of expert e's pairs from
+// that chunk; expert_offsets[e] the first position of the expert. One workgroup.
+__global__ __launch_bounds__(1024) void moe_scan_kernel(int* __restrict__ chunk_hist,
+                                                        int* __restrict__ expert_offsets,
+                                                        int chunks, int n_experts) {
+    extern __shared__ int s_count[];  // [n_experts]
+    for (int e = threadIdx.x; e < n_experts; e += 1024) {
+        int running = 0;
+        for (int c = 0; c < chunks; ++c) {
+            const int v = chunk_hist[(size_t)c * n_experts + e];
+            chunk_hist[(size_t)c * n_experts + e] = running;
+            running += v;
+        }
+        s_count[e] = running;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int running = 0;
+        for (int e = 0; e < n_experts; ++e) {
+            const int v = s_count[e];
+            s_count[e] = running;
+            expert_offsets[e] = running;
+            running += v;
+        }
+        expert_offsets[n_experts] = running;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < n_experts; e += 1024) {
+        const int base = s_count[e];
+        for (int c = 0; c < chunks; ++c) chunk_hist[(size_t)c * n_experts + e] += base;
+    }
+}
+
+// Lane e walks the chunk's pairs in flat order; every pair of expert e takes e's next position.
+__global__ __launch_bounds__(256) void moe_scatter_kernel(const int* __restrict__ ids,
+                                                          const int* __restrict__ chunk_base,
+                                                          int* __restrict__ sorted_pairs,
+                                                          int* __restrict__ pair_pos, int pairs,
+                                                          int pairs_per_chunk, int n_experts) {
+    extern __shared__ int s_ids[];  // [pairs_per_chunk]
+    const int begin = blockIdx.x * pairs_per_chunk;
+    int count = pairs - begin;
+    if (count > pairs_per_chunk) count = pairs_per_chunk;
+    for (int i = threadIdx.x; i < count; i += 256) s_ids[i] = ids[begin + i];
+    __syncthreads();
+    for (int e = threadIdx.x; e < n_experts; e += 256) {
+        int next = chunk_base[(size_t)blockIdx.x * n_experts + e];
+        for (int i = 0; i < count; ++i) {
+            if (s_ids[i] == e) {
+                sorted_pairs[next] = begin + i;
+                pair_pos[begin + i] = next;
+                ++next;
+            }
+        }
+    }
+}
+
+}  // namespace
+
+// ids [tokens, top_k] int32 and weights [tokens, top_k] fp32 from logits [tokens, n_experts] fp32.
+extern "C" void moe_route_launcher(int* ids, float* weights, const float* logits, int tokens,
+                                   int n_experts, int top_k, int config, hipStream_t stream) {
+    (void)config;
+    if (tokens <= 0) return;
+    if (n_experts <= 0 || n_experts > 512 || top_k <= 0 || top_k > 64 || top_k > n_experts) {
+        caa::set_status(CAA_UNSUPPORTED_SHAPE);
+        return;
+    }
+    if (!ids || !weights || !logits) {
+        caa::set_status(CAA_BAD_ARGUMENT);
+        return;
+    }
+    const int blocks = (tokens + 3) / 4;
+    if (n_experts <= 256) {
+        moe_route_kernel<4><<<blocks, 256, 0, stream>>>(logits, ids, weights, tokens, n_experts, top_k);
+    } else {
+        moe_route_kernel<8><<<blocks, 256, 0, stream>>>(logits, ids, weights, tokens, n_experts, top_k);
+    }
+}
+
+// Stable counting sort of the tokens*top_k pairs by expert id.
+//   sorted_pairs[pos] = flat pair index (token*top_k + slot); pair_pos is its inverse;
+//   expert_offsets[e] .. expert_offsets[e+1] are expert e's positions.
+//   chunk_scratch: ceil(tokens/256) * n_experts ints.
+extern "C" void moe_sort_launcher(int* sorted_pairs, int* pair_pos, int* expert_offsets,
+                                  int* chunk_scratch, const int* ids, int tokens, int n_experts,
+                                  int top_k, int config, hipStream_t stream) {
+    (void)config;
+    if (tokens <= 0) return;
+    if (n_experts <= 0 || n_experts > 4096 || top_k <= 0 || top_k > 64) {
+        caa::set_status(CAA_UNSUPPORTED_SHAPE);
+        return;
+    }
+    if (!sorted_pairs || !pair_pos || !expert_offsets || !chunk_scratch || !ids) {
+        caa::set_status(CAA_BAD_ARGUMENT);
+        return;
+    }
+    const int pairs = tokens * top_k;
+    const int pairs_per_chunk = moe::SORT_CHUNK_TOKENS * top_k;
+    const int chunks = (tokens + moe::SORT_CHUNK_TOKENS - 1) / moe::SORT_CHUNK_TOKENS;
+    moe_hist_kernel<<<chunks, 256, n_experts * sizeof(int), stream>>>(ids, chunk_scratch, pairs,
+                                                                     pairs_per_chunk, n_experts);
+    moe_scan_kernel<<<1, 1024, n_experts * sizeof(int), stream>>>(chunk_scratch, expert_offsets, chunks,
+                                                                 n_experts);
+    moe_scatter_kernel<<<chunks, 256, pairs_per_chunk * sizeof(int), stream>>>(
+        ids, chunk_scratch, sorted_pairs, pair_pos, pairs, pairs_per_chunk, n_experts);
+}

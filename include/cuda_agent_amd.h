@@ -96,6 +96,71 @@ int sparse_mla_decode_num_splits(int batch, int n_heads, int topk, int config);
 /* Bytes of workspace sparse_mla_decode_launcher needs for these sizes and this config. */
 size_t sparse_mla_decode_workspace_bytes(int batch, int n_heads, int topk, int config);
 
+/* ---- FP8 block-scaled MoE layer (workload configs 2 and 4 of the benchmark definition;
+ * launcher pattern agent_workdir/kernels/axpby.cu:12-20). Expert weights are e4m3 with one fp32
+ * scale per 128x128 block: w13_q [E, 2*inter, hidden] (rows 0..inter-1 gate, inter..2*inter-1
+ * up), w13_s [E, 2*inter/128, hidden/128], w2_q [E, hidden, inter], w2_s [E, hidden/128,
+ * inter/128]. Activations are quantised per row and 128-wide group:
+ * scale = max(amax, 1e-12)/448, code = e4m3_rne(clamp(v/scale, -448, 448)).
+ * The stages are exported one by one so that a checker can compare each against a reference;
+ * moe_fp8_launcher runs them in sequence. ---- */
+
+/* ids [tokens, top_k] int32: the top_k largest logits of each token, descending, ties to the
+ * lower expert id; weights [tokens, top_k] fp32: sigmoid(logit) normalised over the top_k.
+ * logits [tokens, n_experts] fp32. n_experts <= 512, top_k <= 64. */
+void moe_route_launcher(int* ids, float* weights, const float* logits, int tokens, int n_experts,
+                        int top_k, int config, hipStream_t stream);
+
+/* Stable counting sort of the tokens*top_k (token, slot) pairs by expert id:
+ * sorted_pairs[pos] = token*top_k + slot, pair_pos = its inverse, expert e owns positions
+ * expert_offsets[e] .. expert_offsets[e+1]-1 (expert_offsets has n_experts+1 entries).
+ * chunk_scratch: ceil(tokens/256)*n_experts ints of device scratch. */
+void moe_sort_launcher(int* sorted_pairs, int* pair_pos, int* expert_offsets, int* chunk_scratch,
+                       const int* ids, int tokens, int n_experts, int top_k, int config,
+                       hipStream_t stream);
+
+/* q [rows, cols] e4m3 codes and scales [rows, cols/128] fp32 from x [rows, cols] bf16. */
+void moe_quant_bf16_launcher(void* q, float* scales, const void* x, int rows, int cols, int config,
+                             hipStream_t stream);
+
+/* Grouped gate/up GEMM with SiLU(gate)*up and requantisation fused:
+ * h_q [tokens*top_k, inter] e4m3, h_s [tokens*top_k, inter/128] fp32, rows in sorted order.
+ * config: 0 sizes the pass from the average pairs per expert; 1, 2, 4 force 16, 32, 64 pairs
+ * per pass. */
+void moe_gate_up_launcher(void* h_q, float* h_s, const void* x_q, const float* x_s,
+                          const void* w13_q, const float* w13_s, const int* sorted_pairs,
+                          const int* expert_offsets, int tokens, int hidden, int inter,
+                          int n_experts, int top_k, int config, hipStream_t stream);
+
+/* Grouped down GEMM: y [tokens*top_k, hidden] fp32, rows in sorted order. config as above. */
+void moe_down_launcher(float* y, const void* h_q, const float* h_s, const void* w2_q,
+                       const float* w2_s, const int* expert_offsets, int tokens, int hidden,
+                       int inter, int n_experts, int top_k, int config, hipStream_t stream);
+
+/* out[t, :] = sum_k weights[t, k] * y[pair_pos[t*top_k + k], :], k ascending, in fp32;
+ * out is bf16 (out_dtype 0) or fp32 (out_dtype 1). */
+void moe_combine_launcher(void* out, const float* y, const float* weights, const int* pair_pos,
+                          int tokens, int hidden, int top_k, int out_dtype, int config,
+                          hipStream_t stream);
+
+/* Bytes of device scratch moe_fp8_launcher needs (routing tables, quantised activations,
+ * intermediate h and y). */
+size_t moe_fp8_workspace_bytes(int tokens, int hidden, int inter, int n_experts, int top_k);
+
+/* Byte offsets, inside that workspace, of ids, weights, expert_offsets, sorted_pairs, pair_pos,
+ * x_q, x_s, h_q, h_s, y (in this order), for checkers that inspect the stages. */
+void moe_fp8_workspace_layout(size_t* offsets10, int tokens, int hidden, int inter, int n_experts,
+                              int top_k);
+
+/* The whole layer: out [tokens, hidden] (bf16 if out_dtype == 0, the operator's output type;
+ * fp32 if 1, the same values before the final rounding) from x [tokens, hidden] bf16 and
+ * logits [tokens, n_experts] fp32. workspace: moe_fp8_workspace_bytes(...) bytes, 256-byte
+ * aligned. hidden and inter multiples of 128. config as for moe_gate_up_launcher. */
+void moe_fp8_launcher(void* out, const void* x, const float* logits, const void* w13_q,
+                      const float* w13_s, const void* w2_q, const float* w2_s, void* workspace,
+                      size_t workspace_bytes, int tokens, int hidden, int inter, int n_experts,
+                      int top_k, int out_dtype, int config, hipStream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

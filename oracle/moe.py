@@ -1,0 +1,202 @@
+"""Oracle for the FP8 block-scaled MoE layer (test infrastructure only).
+
+Specification restated (workload configs 2 and 4): ``forward(x[T,H] bf16, logits[T,E] fp32) ->
+out[T,H] bf16`` with expert buffers ``w13_q[E,2I,H]`` e4m3 (rows 0..I-1 gate, I..2I-1 up),
+``w13_s[E,2I/128,H/128]`` fp32, ``w2_q[E,H,I]`` e4m3, ``w2_s[E,H/128,I/128]`` fp32:
+
+  route      s = sigmoid(logits); the 8 experts of a token are its 8 largest logits (ties: the
+             lower expert id), listed in that order; w = s[ids] / sum(s[ids])
+  sort       stable counting sort of the T*8 (token, slot) pairs by expert id
+  quantise   per row and 128-wide group: scale = max(amax, 1e-12)/448,
+             q = e4m3_rne(clamp(v / scale, -448, 448))
+  expert     gu = deq(x_q) @ deq(w13[e]).T ; h = silu(g) * u ; h_q, h_s = quantise(h) ;
+             y = deq(h_q) @ deq(w2[e]).T                    (fp32)
+  combine    out[t] = sum_k w[t,k] * y[t,k], k ascending, fp32 -> bf16
+
+Ranking by logit equals ranking by an exact sigmoid and does not depend on how a particular
+sigmoid implementation rounds. The reference repository has no implementation of this operator;
+only its model contract (agent_workdir/model.py:9-26) shapes the functions below.
+
+Pinned by (tests/test_oracle_moe.py):
+  * e4m3: the 256-entry decode table against torch's float8_e4m3fn and the closed form; the
+    encoder against torch's cast on every representable value, every midpoint and random
+    floats; idempotence; the group maximum maps to +-448;
+  * routing/sort: torch.topk / stable argsort / bincount, brute force on tiny sizes, and the
+    permutation invariants;
+  * GEMMs/combine: float64 dense matmul on dequantised tiny shapes; the exact-integer case;
+    the single-expert (k=1, w=1) case as a plain MLP; block-scale linearity.
+"""
+
+import numpy as np
+import torch
+
+E4M3_MAX = 448.0
+GROUP = 128
+AMAX_FLOOR = 1e-12
+
+
+# ---------------------------------------------------------------------------------- e4m3 codec
+
+def e4m3_decode_table():
+    """float32[256]: value of every OCP e4m3fn code (0x7f / 0xff are NaN), from the closed form."""
+    out = np.zeros(256, dtype=np.float32)
+    for code in range(256):
+        sign = -1.0 if code & 0x80 else 1.0
+        exp = (code >> 3) & 0xF
+        man = code & 0x7
+        if exp == 0xF and man == 0x7:
+            val = np.nan
+        elif exp == 0:
+            val = man * 2.0 ** -9
+        else:
+            val = (1.0 + man / 8.0) * 2.0 ** (exp - 7)
+        out[code] = sign * val
+    return out
+
+
+def e4m3_encode(x):
+    """Round-to-nearest-even encode of a float32 array to e4m3fn codes (uint8), saturating at
+    +-448 (numpy, independent of torch's cast)."""
+    x = np.asarray(x, dtype=np.float32)
+    a = np.minimum(np.abs(x), np.float32(E4M3_MAX)).astype(np.float64)
+    # exponent of the target binade; subnormals share the step 2^-9
+    e = np.floor(np.log2(np.maximum(a, 2.0 ** -20)))
+    e = np.maximum(e, -6.0)
+    step = 2.0 ** (e - 3)
+    qv = np.rint(a / step) * step            # np.rint rounds half to even
+    qv = np.minimum(qv, E4M3_MAX)
+    # value -> code
+    e2 = np.floor(np.log2(np.maximum(qv, 2.0 ** -20)))
+    normal = qv >= 2.0 ** -6
+    exp_field = np.where(normal, e2 + 7, 0).astype(np.int64)
+    man_field = np.where(normal, np.rint((qv / 2.0 ** np.where(normal, e2, 0) - 1.0) * 8),
+                         np.rint(qv * 2.0 ** 9)).astype(np.int64)
+    code = (exp_field << 3) | man_field
+    code = np.where(np.signbit(x), code | 0x80, code)
+    return code.astype(np.uint8)
+
+
+def quantize_groups(v):
+    """Per-row, per-128-group e4m3 quantisation of a 2-D fp32 tensor.
+    Returns (codes float8_e4m3fn [R,C], scales fp32 [R,C/128])."""
+    R, C = v.shape
+    g = v.float().reshape(R, C // GROUP, GROUP)
+    amax = g.abs().amax(dim=-1).clamp_min(AMAX_FLOOR)
+    scale = amax / E4M3_MAX
+    q = (g / scale[:, :, None]).clamp(-E4M3_MAX, E4M3_MAX).to(torch.float8_e4m3fn)
+    return q.reshape(R, C), scale
+
+
+def dequantize_groups(q, scale):
+    R, C = q.shape
+    return (q.float().reshape(R, C // GROUP, GROUP) * scale[:, :, None]).reshape(R, C)
+
+
+def dequantize_blocks(w_q, w_s):
+    """w_q [N,K] e4m3 with one fp32 scale per 128x128 block, w_s [N/128, K/128] -> fp32 [N,K]."""
+    N, K = w_q.shape
+    s = w_s.repeat_interleave(GROUP, 0).repeat_interleave(GROUP, 1)
+    return w_q.float() * s[:N, :K]
+
+
+# ------------------------------------------------------------------------------ routing / sort
+
+def route(logits, top_k=8):
+    """ids int32 [T,k] (descending logit, ties to the lower id), weights fp32 [T,k]."""
+    order = torch.sort(logits, dim=-1, descending=True, stable=True).indices[:, :top_k]
+    score = torch.sigmoid(logits.float()).gather(1, order)
+    return order.int(), score / score.sum(dim=-1, keepdim=True)
+
+
+def sort_pairs(ids, n_experts):
+    """Stable counting sort of the flattened (token, slot) pairs by expert.
+    Returns sorted_pairs int32 [T*k] (flat pair index at each sorted position),
+    pair_pos int32 [T*k] (its inverse) and expert_offsets int32 [E+1]."""
+    flat = ids.reshape(-1).long()
+    sorted_pairs = torch.sort(flat, stable=True).indices
+    counts = torch.bincount(flat, minlength=n_experts)
+    offsets = torch.zeros(n_experts + 1, dtype=torch.long)
+    offsets[1:] = counts.cumsum(0)
+    pair_pos = torch.empty_like(sorted_pairs)
+    pair_pos[sorted_pairs] = torch.arange(flat.numel())
+    return sorted_pairs.int(), pair_pos.int(), offsets.int()
+
+
+# ----------------------------------------------------------------------------------- the layer
+
+def silu(x):
+    return x / (1.0 + torch.exp(-x))
+
+
+def moe_forward(x, logits, w13_q, w13_s, w2_q, w2_s, top_k=8, out_dtype=torch.bfloat16,
+                return_intermediates=False):
+    T, H = x.shape
+    E, I2, _ = w13_q.shape
+    I = I2 // 2
+    ids, weights = route(logits, top_k)
+    x_q, x_s = quantize_groups(x.float())
+    x_dq = dequantize_groups(x_q, x_s)
+    y = torch.zeros(T, top_k, H)
+    h_q_all = torch.zeros(T, top_k, I, dtype=torch.float8_e4m3fn)
+    h_s_all = torch.zeros(T, top_k, I // GROUP)
+    for e in torch.unique(ids).tolist():
+        tok, slot = torch.nonzero(ids == e, as_tuple=True)
+        w13 = dequantize_blocks(w13_q[e], w13_s[e])
+        gu = x_dq[tok] @ w13.T
+        h = silu(gu[:, :I]) * gu[:, I:]
+        h_q, h_s = quantize_groups(h)
+        h_q_all[tok, slot] = h_q
+        h_s_all[tok, slot] = h_s
+        y[tok, slot] = dequantize_groups(h_q, h_s) @ dequantize_blocks(w2_q[e], w2_s[e]).T
+    out = torch.zeros(T, H)
+    for k in range(top_k):
+        out += weights[:, k:k + 1] * y[:, k]
+    out = out.to(out_dtype)
+    if return_intermediates:
+        return out, dict(ids=ids, weights=weights, x_q=x_q, x_s=x_s, h_q=h_q_all, h_s=h_s_all, y=y)
+    return out
+
+
+# ---------------------------------------------------------------------------- synthetic inputs
+
+def random_e4m3(shape, generator=None, device='cpu'):
+    """Uniformly random e4m3 codes with the two NaN codes excluded: magnitudes are log-uniform
+    over the format's range, so a 128-term dot product is dominated by its few largest terms."""
+    codes = torch.randint(0, 256, shape, dtype=torch.uint8, generator=generator, device=device)
+    codes = torch.where((codes & 0x7F) == 0x7F, codes ^ 1, codes)
+    return codes.view(torch.float8_e4m3fn)
+
+
+def normal_e4m3(shape, std, generator=None, device='cpu'):
+    """e4m3 codes of N(0, std) samples, clamped to +-448."""
+    v = torch.randn(shape, generator=generator, device=device) * std
+    return v.clamp(-E4M3_MAX, E4M3_MAX).to(torch.float8_e4m3fn)
+
+
+def moe_make_weights(n_experts, hidden, inter, generator=None, device='cpu'):
+    """Expert weights: e4m3 codes of N(0, 448/sqrt(fan_in)) and 128x128 block scales
+    ~ U(0.5, 1.5)/448, so that a dequantised weight is about N(0, 1/fan_in) and the
+    pre-activations of N(0,1) inputs are O(1). (The workload leaves the code distribution open.)"""
+    gen = generator
+    w13_q = normal_e4m3((n_experts, 2 * inter, hidden), E4M3_MAX / hidden ** 0.5, gen, device)
+    w2_q = normal_e4m3((n_experts, hidden, inter), E4M3_MAX / inter ** 0.5, gen, device)
+    w13_s = (0.5 + torch.rand(n_experts, 2 * inter // GROUP, hidden // GROUP, generator=gen,
+                              device=device)) / 448.0
+    w2_s = (0.5 + torch.rand(n_experts, hidden // GROUP, inter // GROUP, generator=gen,
+                             device=device)) / 448.0
+    return w13_q, w13_s, w2_q, w2_s
+
+
+def moe_make_inputs(tokens, hidden, n_experts, generator=None, device='cpu', biased_experts=None,
+                    bias=2.0):
+    x = torch.randn(tokens, hidden, generator=generator, device=device).bfloat16()
+    logits = torch.randn(tokens, n_experts, generator=generator, device=device)
+    if biased_experts is not None:
+        logits[:, biased_experts] += bias
+    return [x, logits]
+
+
+def rel_rms_error(actual, expected):
+    a = actual.double()
+    e = expected.double()
+    return ((a - e).abs().max() / e.pow(2).mean().sqrt()).item()

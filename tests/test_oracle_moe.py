@@ -1,0 +1,174 @@
+"""Pins the MoE oracle: e4m3 codec, routing/sort, and the GEMM/combine arithmetic."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe
+
+
+def test_decode_table_matches_torch_and_closed_form():
+    tab = moe.e4m3_decode_table()
+    t = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).float().numpy()
+    assert np.array_equal(np.isnan(tab), np.isnan(t))
+    assert np.array_equal(tab[~np.isnan(tab)], t[~np.isnan(t)])
+    assert np.isnan(tab[0x7F]) and np.isnan(tab[0xFF]) and np.isnan(tab).sum() == 2
+    assert tab[0x7E] == 448.0 and tab[0x38] == 1.0 and tab[0x01] == 2.0 ** -9 and tab[0x08] == 2.0 ** -6
+
+
+def test_encoder_matches_torch_cast_on_values_midpoints_and_random():
+    tab = moe.e4m3_decode_table()
+    vals = np.sort(tab[~np.isnan(tab)])
+    mids = (vals[:-1].astype(np.float64) + vals[1:]) / 2
+    rng = np.random.default_rng(0)
+    probe = np.concatenate([vals, mids.astype(np.float32), np.nextafter(mids.astype(np.float32), 1e9),
+                            np.nextafter(mids.astype(np.float32), -1e9),
+                            rng.standard_normal(200000).astype(np.float32) * 100,
+                            rng.standard_normal(50000).astype(np.float32) * 0.01,
+                            np.array([449, 464, 465, 480, 1e6, -1e6, 0.0, -0.0], dtype=np.float32)])
+    got = moe.e4m3_encode(probe)
+    want = torch.from_numpy(probe).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(got, want)
+    # known answers (round half to even, saturation, subnormals)
+    ka = {448.0: 0x7E, 500.0: 0x7E, 17.0: 0x58, 18.0: 0x59, 1.0: 0x38, 0.25: 0x28, 2.0 ** -10: 0x00,
+          3 * 2.0 ** -10: 0x02, 9.7e-4: 0x00, -1.0: 0xB8}
+    for v, code in ka.items():
+        assert moe.e4m3_encode(np.float32(v)) == code, v
+
+
+def test_encode_decode_idempotent():
+    tab = moe.e4m3_decode_table()
+    codes = np.array([c for c in range(256) if (c & 0x7F) != 0x7F], dtype=np.uint8)
+    assert np.array_equal(moe.e4m3_encode(tab[codes]) & 0x7F, codes & 0x7F)
+
+
+def test_group_quantisation_properties():
+    gen = torch.Generator().manual_seed(1)
+    v = torch.randn(6, 384, generator=gen) * 3
+    v[2, 128:256] = 0                                   # an all-zero group
+    q, s = moe.quantize_groups(v)
+    assert q.shape == (6, 384) and s.shape == (6, 3)
+    g = q.float().reshape(6, 3, 128).abs().amax(-1)
+    nonzero = v.reshape(6, 3, 128).abs().amax(-1) > 0
+    assert torch.all(g[nonzero] == 448.0)               # the group maximum maps to +-448
+    assert torch.all(q.float()[2, 128:256] == 0) and s[2, 1] == pytest.approx(1e-12 / 448)
+    back = moe.dequantize_groups(q, s)
+    assert ((back - v).abs() <= v.reshape(6, 3, 128).abs().amax(-1).repeat_interleave(128, 1) / 448 * 16 + 1e-9).all()
+    q2, s2 = moe.quantize_groups(back)                  # idempotent on its own output
+    assert torch.equal(q2.view(torch.uint8), q.view(torch.uint8))
+
+
+def test_routing_against_topk_and_brute_force():
+    gen = torch.Generator().manual_seed(2)
+    logits = torch.randn(50, 256, generator=gen)
+    ids, w = moe.route(logits)
+    vals, idx = torch.topk(logits, 8, dim=-1)           # distinct floats: same order
+    assert torch.equal(ids.long(), idx)
+    torch.testing.assert_close(w.sum(-1), torch.ones(50))
+    s = torch.sigmoid(vals)
+    torch.testing.assert_close(w, s / s.sum(-1, keepdim=True))
+    for t in range(5):                                  # brute force
+        order = sorted(range(256), key=lambda e: (-logits[t, e].item(), e))[:8]
+        assert ids[t].tolist() == order
+    assert all(len(set(r)) == 8 for r in ids.tolist())
+
+
+def test_routing_ties_go_to_lower_id():
+    logits = torch.zeros(2, 16)
+    logits[0, [3, 9, 12]] = 1.0
+    logits[1, 5] = -0.0
+    ids, _ = moe.route(logits, top_k=4)
+    assert ids[0].tolist() == [3, 9, 12, 0] and ids[1].tolist() == [0, 1, 2, 3]
+
+
+def test_sort_is_a_stable_counting_sort():
+    gen = torch.Generator().manual_seed(3)
+    ids, _ = moe.route(torch.randn(300, 32, generator=gen), top_k=4)
+    sp, pos, off = moe.sort_pairs(ids, 32)
+    flat = ids.reshape(-1)
+    assert sorted(sp.tolist()) == list(range(1200))
+    assert torch.equal(pos[sp.long()].long(), torch.arange(1200))
+    assert off[0] == 0 and off[-1] == 1200
+    assert torch.equal((off[1:] - off[:-1]).long(), torch.bincount(flat.long(), minlength=32))
+    for e in range(32):
+        seg = sp[off[e]:off[e + 1]]
+        assert torch.all(flat[seg.long()] == e)
+        assert torch.all(seg[1:] > seg[:-1])            # stable: ascending flat pair index
+
+
+def _tiny(seed=4, E=4, H=256, I=128, T=8):
+    gen = torch.Generator().manual_seed(seed)
+    w = moe.moe_make_weights(E, H, I, gen)
+    x, logits = moe.moe_make_inputs(T, H, E, gen)
+    return x, logits, w
+
+
+def test_layer_against_float64_dense():
+    x, logits, (w13_q, w13_s, w2_q, w2_s) = _tiny()
+    out, mid = moe.moe_forward(x, logits, w13_q, w13_s, w2_q, w2_s, top_k=2, out_dtype=torch.float32,
+                               return_intermediates=True)
+    ids, wts = mid['ids'], mid['weights'].double()
+    xd = moe.dequantize_groups(mid['x_q'], mid['x_s']).double()
+    want = torch.zeros(8, 256, dtype=torch.float64)
+    for t in range(8):
+        for k in range(2):
+            e = ids[t, k].item()
+            gu = moe.dequantize_blocks(w13_q[e], w13_s[e]).double() @ xd[t]
+            h = gu[:128] / (1 + torch.exp(-gu[:128])) * gu[128:]
+            hq, hs = moe.quantize_groups(h.float()[None])
+            want[t] += wts[t, k] * (moe.dequantize_blocks(w2_q[e], w2_s[e]).double()
+                                    @ moe.dequantize_groups(hq, hs)[0].double())
+    assert moe.rel_rms_error(out, want) < 1e-4
+
+
+def test_exact_integer_case():
+    # scales 1, small-integer codes, zero logits except the winners: every partial sum is an
+    # exactly representable integer, so fp32 evaluation order cannot matter.
+    E, H, I, T = 2, 128, 128, 4
+    gen = torch.Generator().manual_seed(5)
+    w13 = torch.randint(-2, 3, (E, 2 * I, H), generator=gen).float()
+    w2 = torch.randint(-2, 3, (E, H, I), generator=gen).float()
+    x = torch.randint(-3, 4, (T, H), generator=gen).float()
+    x[:, 0] = 448.0                                     # amax 448 -> activation scale exactly 1
+    xq, xs = moe.quantize_groups(x)
+    assert torch.all(xs == 1.0) and torch.equal(xq.float(), x)
+    gu = x @ w13[0].T
+    assert torch.equal(gu, (x.double() @ w13[0].double().T).float())
+
+
+def test_single_expert_is_a_plain_mlp():
+    x, logits, (w13_q, w13_s, w2_q, w2_s) = _tiny(6, E=1, T=5)
+    out = moe.moe_forward(x, logits, w13_q, w13_s, w2_q, w2_s, top_k=1, out_dtype=torch.float32)
+    xq, xs = moe.quantize_groups(x.float())
+    gu = moe.dequantize_groups(xq, xs) @ moe.dequantize_blocks(w13_q[0], w13_s[0]).T
+    h = moe.silu(gu[:, :128]) * gu[:, 128:]
+    hq, hs = moe.quantize_groups(h)
+    want = moe.dequantize_groups(hq, hs) @ moe.dequantize_blocks(w2_q[0], w2_s[0]).T
+    torch.testing.assert_close(out, want, rtol=1e-6, atol=1e-6)
+
+
+def test_block_scale_acts_on_its_k_slice_only():
+    x, logits, (w13_q, w13_s, w2_q, w2_s) = _tiny(7, E=1, T=3)
+    xq, xs = moe.quantize_groups(x.float())
+    xd = moe.dequantize_groups(xq, xs)
+    base = xd @ moe.dequantize_blocks(w13_q[0], w13_s[0]).T
+    s2 = w13_s.clone()
+    s2[0, 1, 0] *= 3.0                                  # rows 128..255, K columns 0..127
+    bumped = xd @ moe.dequantize_blocks(w13_q[0], s2[0]).T
+    delta = 2.0 * (xd[:, :128] @ moe.dequantize_blocks(w13_q[0], w13_s[0])[128:256, :128].T)
+    torch.testing.assert_close(bumped[:, 128:256] - base[:, 128:256], delta, rtol=1e-4, atol=1e-4)
+    assert torch.equal(bumped[:, :128], base[:, :128])
+
+
+def test_silu_closed_form():
+    v = torch.linspace(-20, 20, 101)
+    torch.testing.assert_close(moe.silu(v), torch.nn.functional.silu(v), rtol=1e-6, atol=1e-7)
+    assert moe.silu(torch.tensor(0.0)) == 0
+
+
+def test_weight_generator_has_no_nan_codes():
+    gen = torch.Generator().manual_seed(8)
+    w13_q, w13_s, w2_q, w2_s = moe.moe_make_weights(2, 256, 128, gen)
+    for q in (w13_q, w2_q, moe.random_e4m3((1000,), gen)):
+        assert ((q.view(torch.uint8) & 0x7F) != 0x7F).all()
+    assert (w13_s > 0.5 / 448 - 1e-9).all() and (w13_s < 1.5 / 448 + 1e-9).all()
+    assert w13_s.shape == (2, 2, 2) and w2_s.shape == (2, 2, 1)
