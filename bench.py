@@ -1,0 +1,268 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X: each workload of the benchmark definition run through
+the C-ABI library on synthetic, HBM-resident inputs, timed with HIP events on the launch stream.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workloads gdn,moe_decode,mla,moe_prefill]
+                    [--no-cpu-baseline]
+
+Prints ONE JSON line. The headline (`metric`/`value`/`roofline`/`cpu_baseline`) is workload
+configs[1], the batched GDN decode step; the other single-GPU workloads are reported under
+`workloads` with the same fields. A "step" is one launch of the operator on one batch.
+
+Algorithmic work per launch (what `roofline.achieved` is computed from):
+  gdn          2*B*Hv*dk*dv*4 (state read + write) + q,k,v,g,beta,o        = 1 082 195 968 B
+  moe_decode   n_active*(44 040 192 + 10 752) + x + logits + out           (n_active measured)
+  mla          B*topk*576*2 gathered bytes                                  =   150 994 944 B
+  moe_prefill  T*8*(2*H*2I + 2*I*H) flop                                    = 5.772e12 flop
+Inputs that fit the 256 MB last-level cache are rotated over several sets so that repeated steps
+do not read from cache what the workload would read from HBM.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+REPO = Path(__file__).resolve().parent
+if str(REPO) not in sys.path:
+    sys.path.insert(0, str(REPO))
+
+HBM_PEAK_GBS = 8000.0
+FP8_PEAK_TFLOPS = 5033.0
+METRIC = "GB/s & % HBM peak (GDN/MoE/MLA decode); fp8 TFLOP/s % MFMA peak (MoE prefill)"
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (profiles/*_pmc.txt), scaled by the same counters read on a plain copy kernel; None = not measured.
+MEASURED_TRAFFIC = {'gdn': None, 'moe_decode': None, 'mla': None, 'moe_prefill': None}
+
+
+def timed_launches(torch, launch, steps, warmup):
+    """Average device time of one launch in seconds, HIP events on the current (launch) stream."""
+    for i in range(warmup):
+        launch(i)
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(steps):
+        launch(warmup + i)
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) * 1e-3 / steps
+
+
+def cpu_time(fn, min_seconds=3.0, max_iters=5):
+    fn()  # warm-up
+    t0 = time.perf_counter()
+    n = 0
+    while n < max_iters and (n == 0 or time.perf_counter() - t0 < min_seconds):
+        fn()
+        n += 1
+    return (time.perf_counter() - t0) / n
+
+
+def bench_gdn(torch, capi, dev, steps, warmup, cpu_baseline):
+    from oracle import gdn
+    B, Hv, Hqk = 256, 32, 16
+    gen = torch.Generator(device=dev).manual_seed(20251)
+    sets = []
+    for _ in range(3):  # 3 x 537 MB of state: each step streams a set the cache no longer holds
+        q = torch.randn(B, Hqk, 128, device=dev, generator=gen)
+        k = torch.randn(B, Hqk, 128, device=dev, generator=gen)
+        q = (q / q.norm(dim=-1, keepdim=True)).bfloat16()
+        k = (k / k.norm(dim=-1, keepdim=True)).bfloat16()
+        v = torch.randn(B, Hv, 128, device=dev, generator=gen).bfloat16()
+        g = torch.exp(-0.5 * torch.log1p(torch.exp(torch.randn(B, Hv, device=dev, generator=gen))))
+        beta = torch.sigmoid(torch.randn(B, Hv, device=dev, generator=gen))
+        state = 0.02 * torch.randn(B, Hv, 128, 128, device=dev, generator=gen)
+        o = torch.empty(B, Hv, 128, device=dev)
+        sets.append((o, state, q, k, v, g, beta))
+    sec = timed_launches(torch, lambda i: capi.gdn_decode_launch(*sets[i % 3]), steps, warmup)
+    work = 2 * B * Hv * 128 * 128 * 4 + 2 * B * Hqk * 128 * 2 + B * Hv * 128 * 2 + 2 * B * Hv * 4 + B * Hv * 128 * 4
+    res = dict(
+        workload="configs[1]: GDN batched decode B=256, Hv=32/Hqk=16 (GQA 2:1), dk=dv=128, bf16 q/k/v, "
+                 "fp32 state 537 MB updated in place, seed 20251",
+        value=work / sec / 1e9, unit="GB/s", ms_per_step=sec * 1e3, dtype="f32", kernel="gdn_decode_kernel",
+        roofline=dict(bound="hbm", achieved=work / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
+                      frac=work / sec / 1e9 / HBM_PEAK_GBS, traffic=MEASURED_TRAFFIC['gdn']),
+        algorithmic_bytes=work)
+    if cpu_baseline:
+        cores = len(os.sched_getaffinity(0))
+        torch.set_num_threads(cores)
+        cgen = torch.Generator().manual_seed(20251)
+        ins = gdn.gdn_make_inputs(B, Hv, Hqk, qkv_dtype=torch.bfloat16, generator=cgen)
+        csec = cpu_time(lambda: gdn.gdn_decode_step(*ins))
+        res['cpu_baseline'] = dict(value=work / csec / 1e9, unit="GB/s", cores=cores, kind="port",
+                                   sample="the full configs[1] step (eager PyTorch oracle, state in place), "
+                                          "1 warm-up + up to 5 timed steps")
+    return res
+
+
+def bench_mla(torch, capi, dev, steps, warmup, cpu_baseline):
+    from oracle import mla
+    B, H, N, topk = 64, 128, 32768, 2048
+    gen = torch.Generator(device=dev).manual_seed(20253)
+    q = torch.randn(B, H, 576, device=dev, generator=gen).bfloat16()
+    kv = torch.randn(B, N, 576, device=dev, generator=gen).bfloat16()
+    # 4 index sets: the 151 MB gathered by one step would otherwise be served from the cache
+    idxs = [torch.stack([torch.randperm(N, device=dev, generator=gen)[:topk] for _ in range(B)]).int()
+            for _ in range(4)]
+    out = torch.empty(B, H, 512, device=dev, dtype=torch.bfloat16)
+    ws = torch.empty(capi.sparse_mla_workspace_bytes(B, H, topk), dtype=torch.uint8, device=dev)
+    sec = timed_launches(torch, lambda i: capi.sparse_mla_decode_launch(out, q, kv, idxs[i % 4], ws), steps, warmup)
+    work = B * topk * 576 * 2
+    flops = 2 * B * H * topk * (576 + 512)
+    res = dict(
+        workload="configs[3]: sparse-MLA decode B=64, 128 heads, 576-dim latent rows, top-k 2048 of 32768, "
+                 "bf16, seed 20253 (split kernel + merge per step)",
+        value=work / sec / 1e9, unit="GB/s", ms_per_step=sec * 1e3, dtype="bf16", kernel="sparse_mla_split_kernel",
+        roofline=dict(bound="hbm", achieved=work / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
+                      frac=work / sec / 1e9 / HBM_PEAK_GBS, traffic=MEASURED_TRAFFIC['mla']),
+        algorithmic_bytes=work, tflops=flops / sec / 1e12)
+    if cpu_baseline:
+        cores = len(os.sched_getaffinity(0))
+        torch.set_num_threads(cores)
+        nb = 8
+        cq, ckv, cidx = q[:nb].cpu(), kv[:nb].cpu(), idxs[0][:nb].cpu()
+        csec = cpu_time(lambda: mla.sparse_mla_decode(cq, ckv, cidx))
+        res['cpu_baseline'] = dict(value=nb * topk * 576 * 2 / csec / 1e9, unit="GB/s", cores=cores, kind="port",
+                                   sample="requests 0..7 of configs[3] (1/8 of the batch), eager PyTorch oracle")
+    return res
+
+
+def make_moe(torch, dev, tokens, biased):
+    H, I, E = 7168, 2048, 256
+    gen = torch.Generator(device=dev).manual_seed(20252 if not biased else 20254)
+    w13_q = torch.empty(E, 2 * I, H, dtype=torch.float8_e4m3fn, device=dev)
+    w2_q = torch.empty(E, H, I, dtype=torch.float8_e4m3fn, device=dev)
+    for e in range(E):
+        w13_q[e] = (torch.randn(2 * I, H, device=dev, generator=gen) * (448 / H ** 0.5)).to(torch.float8_e4m3fn)
+        w2_q[e] = (torch.randn(H, I, device=dev, generator=gen) * (448 / I ** 0.5)).to(torch.float8_e4m3fn)
+    w13_s = (0.5 + torch.rand(E, 2 * I // 128, H // 128, device=dev, generator=gen)) / 448
+    w2_s = (0.5 + torch.rand(E, H // 128, I // 128, device=dev, generator=gen)) / 448
+    x = torch.randn(tokens, H, device=dev, generator=gen).bfloat16()
+    logits = torch.randn(tokens, E, device=dev, generator=gen)
+    if biased:
+        logits[:, torch.randperm(E, device=dev, generator=gen)[:16]] += 2.0
+    return x, logits, w13_q, w13_s, w2_q, w2_s
+
+
+def moe_cpu_baseline(torch, tensors, n_tokens):
+    from oracle import moe
+    cores = len(os.sched_getaffinity(0))
+    torch.set_num_threads(cores)
+    x, logits, w13_q, w13_s, w2_q, w2_s = tensors
+    ids, _ = moe.route(logits[:n_tokens].cpu(), 8)
+    used = torch.unique(ids).tolist()
+    remap = {e: i for i, e in enumerate(used)}
+    sub = torch.full((n_tokens, len(used)), -30.0)
+    for t in range(n_tokens):
+        for e in ids[t].tolist():
+            sub[t, remap[e]] = logits[t, e].item()
+    sel = torch.tensor(used, device=x.device)
+    host = [t.cpu() for t in (x[:n_tokens], )] + [sub] + [t[sel].cpu() for t in (w13_q, w13_s, w2_q, w2_s)]
+    csec = cpu_time(lambda: moe.moe_forward(*host, top_k=8), min_seconds=2.0, max_iters=2)
+    return csec, len(used), cores
+
+
+def bench_moe(torch, capi, dev, steps, warmup, cpu_baseline, prefill):
+    T = 8192 if prefill else 64
+    H, I, E, k = 7168, 2048, 256, 8
+    tensors = make_moe(torch, dev, T, prefill)
+    x, logits, w13_q, w13_s, w2_q, w2_s = tensors
+    ws = torch.empty(capi.moe_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device=dev)
+    out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    sec = timed_launches(torch, lambda i: capi.moe_fp8_launch(out, x, logits, w13_q, w13_s, w2_q, w2_s, ws),
+                         steps, warmup)
+    off = capi.moe_workspace_views(ws, T, H, I, E, k)['expert_offsets'].cpu()
+    n_active = int(((off[1:] - off[:-1]) > 0).sum())
+    flops = T * k * (2 * H * 2 * I + 2 * I * H)
+    wbytes = n_active * (3 * I * H + (3 * I * H // (128 * 128)) * 4) + T * H * 2 + T * E * 4 + T * H * 2
+    if prefill:
+        res = dict(
+            workload="configs[4]: FP8 MoE prefill T=8192, hidden 7168, 256 experts x inter 2048, top-8, +2 logit "
+                     "bias on 16 experts, e4m3 with 128x128 block scales, seed 20254 (whole layer per step)",
+            value=flops / sec / 1e12, unit="TFLOP/s", ms_per_step=sec * 1e3, dtype="f8e4m3",
+            kernel="moe_stream_gemm_kernel",
+            roofline=dict(bound="mfma", achieved=flops / sec / 1e12, peak=FP8_PEAK_TFLOPS, unit="TFLOP/s",
+                          frac=flops / sec / 1e12 / FP8_PEAK_TFLOPS, traffic=MEASURED_TRAFFIC['moe_prefill']),
+            algorithmic_flops=flops, active_experts=n_active)
+    else:
+        res = dict(
+            workload="configs[2]: FP8 MoE decode T=64, hidden 7168, 256 experts x inter 2048, top-8, e4m3 with "
+                     "128x128 block scales, seed 20252 (whole layer per step)",
+            value=wbytes / sec / 1e9, unit="GB/s", ms_per_step=sec * 1e3, dtype="f8e4m3",
+            kernel="moe_stream_gemm_kernel",
+            roofline=dict(bound="hbm", achieved=wbytes / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
+                          frac=wbytes / sec / 1e9 / HBM_PEAK_GBS, traffic=MEASURED_TRAFFIC['moe_decode']),
+            algorithmic_bytes=wbytes, active_experts=n_active, tflops=flops / sec / 1e12)
+    if cpu_baseline:
+        n_tok = 4
+        csec, n_used, cores = moe_cpu_baseline(torch, tensors, n_tok)
+        if prefill:
+            cval = n_tok * k * (2 * H * 2 * I + 2 * I * H) / csec / 1e12
+        else:
+            cval = (n_used * (3 * I * H + (3 * I * H // (128 * 128)) * 4)) / csec / 1e9
+        res['cpu_baseline'] = dict(
+            value=cval, unit=res['unit'], cores=cores, kind="port",
+            sample=f"tokens 0..{n_tok - 1} of the workload and the {n_used} experts they route to, eager "
+                   "PyTorch oracle (dequantise to fp32, dense matmul)")
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=20)
+    ap.add_argument('--warmup', type=int, default=5)
+    ap.add_argument('--workloads', default='gdn,moe_decode,mla,moe_prefill')
+    ap.add_argument('--no-cpu-baseline', action='store_true')
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit('bench.py: this build measures one GPU only (no collectives, no sharding); run with --gpus 1')
+
+    import torch
+    import __graft_entry__
+    __graft_entry__.load_package()
+    from cuda_agent_amd import capi
+    capi.library()  # raises if the HIP library is not built: there is no fallback path
+    if not torch.cuda.is_available():
+        sys.exit('bench.py: no GPU visible')
+    dev = torch.device('cuda:0')
+    torch.cuda.set_device(dev)
+    cpu = not args.no_cpu_baseline
+    wanted = [w.strip() for w in args.workloads.split(',') if w.strip()]
+    results = {}
+    for name in wanted:
+        if name == 'gdn':
+            results[name] = bench_gdn(torch, capi, dev, args.steps, args.warmup, cpu)
+        elif name == 'mla':
+            results[name] = bench_mla(torch, capi, dev, args.steps, args.warmup, cpu)
+        elif name == 'moe_decode':
+            results[name] = bench_moe(torch, capi, dev, args.steps, args.warmup, cpu, prefill=False)
+        elif name == 'moe_prefill':
+            results[name] = bench_moe(torch, capi, dev, max(2, args.steps // 4), max(1, args.warmup // 2), cpu,
+                                      prefill=True)
+        else:
+            sys.exit(f'bench.py: unknown workload {name}')
+        torch.cuda.empty_cache()
+
+    head_name = 'gdn' if 'gdn' in results else wanted[0]
+    head = results[head_name]
+    line = {
+        "metric": METRIC, "value": head['value'], "unit": head['unit'], "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": head['ms_per_step'], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": head['dtype'], "data": "synthetic",
+        "config": {"workload": head['workload']},
+        "roofline": head['roofline'],
+    }
+    if 'cpu_baseline' in head:
+        line["cpu_baseline"] = head['cpu_baseline']
+    line["workloads"] = {k: v for k, v in results.items() if k != head_name}
+    print(json.dumps(line))
+
+
+if __name__ == '__main__':
+    main()

@@ -9,7 +9,8 @@ namespace moe {
 
 constexpr int GROUP = 128;            // quantisation group along K, and weight block edge
 constexpr float E4M3_MAX = 448.f;
-constexpr float AMAX_FLOOR = 1e-12f;  // scale of an all-zero group: 1e-12 / 448
+constexpr float INV_E4M3_MAX = (float)(1.0 / 448.0);  // scales are amax times this, rounded once
+constexpr float AMAX_FLOOR = 1e-12f;  // an all-zero group gets the scale 1e-12 * fp32(1/448)
 constexpr int SORT_CHUNK_TOKENS = 256;
 
 // Device scratch of one forward pass, carved from the caller's workspace.

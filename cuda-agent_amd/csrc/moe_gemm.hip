@@ -163,7 +163,7 @@ __global__ __launch_bounds__(256) void moe_stream_gemm_kernel(
                 const int idx = nt * 16 + col;
                 const float amax =
                     fmaxf(fmaxf(s_amax[0][idx], s_amax[1][idx]), fmaxf(s_amax[2][idx], s_amax[3][idx]));
-                const float scale = fmaxf(amax, AMAX_FLOOR) / E4M3_MAX;
+                const float scale = fmaxf(amax, AMAX_FLOOR) * INV_E4M3_MAX;
                 if (pos[nt] < end) {
 #pragma unroll
                     for (int i = 0; i < 2; ++i) {

@@ -1,5 +1,5 @@
 // Activation quantisation: bf16 rows -> e4m3 codes with one fp32 scale per 128-wide group.
-//   scale = max(amax, 1e-12) / 448;  code = e4m3_rne(clamp(v / scale, -448, 448))
+//   scale = max(amax, 1e-12) * fp32(1/448);  code = e4m3_rne(clamp(v / scale, -448, 448))
 // One wavefront per (row, group), two elements per lane. The division is IEEE fp32 so that the
 // codes are bit-identical to a CPU evaluation of the same formula; v_cvt_pk_fp8_f32 rounds to
 // nearest even but does not saturate (465 -> NaN), hence the clamp.
@@ -25,7 +25,7 @@ __global__ __launch_bounds__(256) void moe_quant_bf16_kernel(const __hip_bfloat1
     float amax = fmaxf(fabsf(v0), fabsf(v1));
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
-    const float scale = fmaxf(amax, AMAX_FLOOR) / E4M3_MAX;
+    const float scale = fmaxf(amax, AMAX_FLOOR) * INV_E4M3_MAX;
     const float a = fminf(fmaxf(v0 / scale, -E4M3_MAX), E4M3_MAX);
     const float b = fminf(fmaxf(v1 / scale, -E4M3_MAX), E4M3_MAX);
     const int packed = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);

@@ -101,7 +101,7 @@ size_t sparse_mla_decode_workspace_bytes(int batch, int n_heads, int topk, int c
  * scale per 128x128 block: w13_q [E, 2*inter, hidden] (rows 0..inter-1 gate, inter..2*inter-1
  * up), w13_s [E, 2*inter/128, hidden/128], w2_q [E, hidden, inter], w2_s [E, hidden/128,
  * inter/128]. Activations are quantised per row and 128-wide group:
- * scale = max(amax, 1e-12)/448, code = e4m3_rne(clamp(v/scale, -448, 448)).
+ * scale = max(amax, 1e-12) * fp32(1/448), code = e4m3_rne(clamp(v/scale, -448, 448)).
  * The stages are exported one by one so that a checker can compare each against a reference;
  * moe_fp8_launcher runs them in sequence. ---- */
 

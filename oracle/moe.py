@@ -7,8 +7,12 @@ out[T,H] bf16`` with expert buffers ``w13_q[E,2I,H]`` e4m3 (rows 0..I-1 gate, I.
   route      s = sigmoid(logits); the 8 experts of a token are its 8 largest logits (ties: the
              lower expert id), listed in that order; w = s[ids] / sum(s[ids])
   sort       stable counting sort of the T*8 (token, slot) pairs by expert id
-  quantise   per row and 128-wide group: scale = max(amax, 1e-12)/448,
+  quantise   per row and 128-wide group: scale = max(amax, 1e-12) * fp32(1/448),
              q = e4m3_rne(clamp(v / scale, -448, 448))
+             (a multiply by the rounded reciprocal, not a division by 448: eager PyTorch
+             evaluates `tensor / 448.0` that way on the GPU but not on the CPU, and with bf16
+             inputs v/scale often sits exactly on a rounding tie, where one ulp of the scale
+             decides the code)
   expert     gu = deq(x_q) @ deq(w13[e]).T ; h = silu(g) * u ; h_q, h_s = quantise(h) ;
              y = deq(h_q) @ deq(w2[e]).T                    (fp32)
   combine    out[t] = sum_k w[t,k] * y[t,k], k ascending, fp32 -> bf16
@@ -82,7 +86,7 @@ def quantize_groups(v):
     R, C = v.shape
     g = v.float().reshape(R, C // GROUP, GROUP)
     amax = g.abs().amax(dim=-1).clamp_min(AMAX_FLOOR)
-    scale = amax / E4M3_MAX
+    scale = amax * (1.0 / E4M3_MAX)
     q = (g / scale[:, :, None]).clamp(-E4M3_MAX, E4M3_MAX).to(torch.float8_e4m3fn)
     return q.reshape(R, C), scale
 

@@ -8,6 +8,11 @@ element by up to 2^-9 of its magnitude, which for the heavy-tailed outputs of th
 2e-2 rms plus that floor, measured on the reference itself.
 The gather is exact (indices are used verbatim), which the 'equal value rows' and 'only selected
 rows are read' cases check bit for bit."""
+import os
+import subprocess
+import sys
+from pathlib import Path
+
 import pytest
 import torch
 
@@ -148,3 +153,15 @@ def test_rejects_unsupported_shapes(capi, dev):
     out = torch.zeros(1, 128, 512, device=dev, dtype=torch.bfloat16)
     with pytest.raises(capi.LaunchRejected, match='workspace too small'):
         capi.sparse_mla_decode_launch(out, q, kv, idx, ws[:64])
+
+
+@pytest.mark.parametrize('ws_config', ['small', '3'])
+def test_workspace_verification_flow(ws_config):
+    """`python3 -m utils.verification` from inside the workspace, as its user runs it."""
+    ws = Path(__file__).resolve().parent.parent / 'cuda-agent_amd' / 'workspaces' / 'sparse_mla'
+    assert (ws / 'cuda_extension.so').exists(), 'workspace extension not built'
+    env = dict(os.environ, MLA_CONFIG=ws_config)
+    out = subprocess.run([sys.executable, '-m', 'utils.verification'], cwd=ws, env=env,
+                         capture_output=True, text=True, timeout=900)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert '[PASS] check 5/5' in out.stdout and '[PASS] verify success' in out.stdout
