@@ -33,9 +33,11 @@ HBM_PEAK_GBS = 8000.0
 FP8_PEAK_TFLOPS = 5033.0
 METRIC = "GB/s & % HBM peak (GDN/MoE/MLA decode); fp8 TFLOP/s % MFMA peak (MoE prefill)"
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/*_pmc.txt), scaled by the same counters read on a plain copy kernel; None = not measured.
-MEASURED_TRAFFIC = {'gdn': None, 'moe_decode': None, 'mla': None, 'moe_prefill': None}
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled
+# by the same counters read on a plain 512 MiB copy kernel (FETCH_SIZE x 1.99982, WRITE_SIZE x 1,
+# both in KiB); the counter summary is profiles/gdn_mla_moe_decode_hbm_traffic_pmc.md.
+# None = not measured.
+MEASURED_TRAFFIC = {'gdn': 1086009000, 'moe_decode': 6703896000, 'mla': 259339000, 'moe_prefill': None}
 
 
 def timed_launches(torch, launch, steps, warmup):
@@ -219,6 +221,9 @@ def main():
     ap.add_argument('--warmup', type=int, default=5)
     ap.add_argument('--workloads', default='gdn,moe_decode,mla,moe_prefill')
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--calibrate-copy', action='store_true',
+                    help='also run 3 plain device copies of 536 870 912 bytes (a kernel of known traffic, '
+                         'for scaling the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)')
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py: this build measures one GPU only (no collectives, no sharding); run with --gpus 1')
@@ -233,6 +238,13 @@ def main():
     dev = torch.device('cuda:0')
     torch.cuda.set_device(dev)
     cpu = not args.no_cpu_baseline
+    if args.calibrate_copy:
+        src = torch.ones(536870912 // 4, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     wanted = [w.strip() for w in args.workloads.split(',') if w.strip()]
     results = {}
     for name in wanted:
