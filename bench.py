@@ -37,7 +37,7 @@ METRIC = "GB/s & % HBM peak (GDN/MoE/MLA decode); fp8 TFLOP/s % MFMA peak (MoE p
 # by the same counters read on a plain 512 MiB copy kernel (FETCH_SIZE x 1.99982, WRITE_SIZE x 1,
 # both in KiB); the counter summary is profiles/gdn_mla_moe_decode_hbm_traffic_pmc.md.
 # None = not measured.
-MEASURED_TRAFFIC = {'gdn': 1086009000, 'moe_decode': 6703896000, 'mla': 259339000, 'moe_prefill': None}
+MEASURED_TRAFFIC = {'gdn': 1086006640, 'moe_decode': 6703804038, 'mla': 259340846, 'moe_prefill': None}
 
 
 def timed_launches(torch, launch, steps, warmup):
