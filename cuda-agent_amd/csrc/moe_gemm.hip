@@ -196,6 +196,255 @@ __global__ __launch_bounds__(256) void moe_stream_gemm_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Streaming form, LDS-staged (the decode path).
+//
+// Loading the MFMA operand directly makes every load instruction touch 64-byte half lines of 16
+// different rows, and that access pattern was measured to saturate at 5.3 TB/s on this part,
+// against 6.9 TB/s as soon as each instruction covers whole 128-byte lines. Here the weights
+// (and the activations) are therefore brought in by global->LDS loads of 16 bytes per lane in
+// which the 8 lanes of a row fetch one full 128-byte line, and the operands are then read from
+// LDS in the MFMA layout. Every wavefront stages only the rows it consumes itself (4 tiles of 16
+// weight rows, and its own copy of the 16*NT activation rows), so the K loop needs no
+// workgroup barrier: a wavefront waits on its own load counter only. A ring of DEPTH stages of one
+// 128-block each keeps DEPTH-1 blocks (~40 KB per block and workgroup) in flight.
+//
+// LDS slot of the 16-byte chunk c of row r in a 16x128-byte tile: r*8 + (c ^ (r & 7)); the 8
+// lanes that read chunk g of rows 0..7 (or 8..15) then hit 8 different bank groups.
+// A workgroup covers 256 output rows: 128 gate + 128 up rows (GATE_UP), or 256 rows of w2.
+// ---------------------------------------------------------------------------------------------
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit field");
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+    asm volatile("" ::: "memory");  // LDS reads below must not be moved above the wait
+}
+
+// 64 lanes x 16 bytes: global (base + per-lane byte offset) -> LDS (lds_base + lane*16).
+// An asm statement, so the loads stay outside the compiler's bookkeeping of outstanding memory
+// operations; their completion is awaited explicitly with wait_vmcnt<>().
+__device__ __forceinline__ void dma16(const void* base, uint32_t lane_byte_offset, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(lane_byte_offset), "s"(base), "s"(lds_base)
+                 : "memory", "m0");
+}
+__device__ __forceinline__ void dma16_ptr(const void* lane_ptr, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(lane_ptr), "s"(lds_base)
+                 : "memory", "m0");
+}
+
+template <bool GATE_UP, int NT>
+__global__ __launch_bounds__(256) void moe_stream_gemm_lds_kernel(
+    const uint8_t* __restrict__ w_q, const float* __restrict__ w_s, const uint8_t* __restrict__ a_q,
+    const float* __restrict__ a_s, const int* __restrict__ sorted_pairs,
+    const int* __restrict__ expert_offsets, uint8_t* __restrict__ h_q, float* __restrict__ h_s,
+    float* __restrict__ y, int K, int n_rows, int inter, int top_k) {
+    constexpr int TILES = 4;
+    constexpr int DEPTH = 3;
+    constexpr int TILE_BYTES = 16 * GROUP;                       // 2 KB
+    constexpr int STAGE_BYTES = (TILES + NT) * TILE_BYTES;       // per wavefront
+    constexpr int PER_STAGE = 2 * (TILES + NT);                  // load instructions per stage
+    constexpr int MAX_KB = 64;
+    __shared__ __attribute__((aligned(16))) uint8_t s_ring[4 * DEPTH * STAGE_BYTES];
+    __shared__ float s_bscale[MAX_KB][NT * 16];
+    __shared__ float s_amax[4][NT * 16];
+
+    const int e = blockIdx.y;
+    const int rb = blockIdx.x;  // block of 256 output rows (GATE_UP: 128 gate + 128 up)
+    const int begin = expert_offsets[e];
+    const int end = expert_offsets[e + 1];
+    if (end <= begin) return;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int col = lane & 15;
+    const int g = lane >> 4;
+    const int KB = K / GROUP;
+    const int row_blocks = n_rows / GROUP;
+
+    // first weight row of each of this wavefront's tiles, and the scale rows they belong to
+    const uint8_t* tile_base[TILES];
+    const float* ws_ptr[2];
+    if (GATE_UP) {
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) {
+            const int row = (t >> 1) * inter + rb * GROUP + wave * 32 + (t & 1) * 16;
+            tile_base[t] = w_q + ((size_t)e * n_rows + row) * K;
+        }
+        ws_ptr[0] = w_s + ((size_t)e * row_blocks + rb) * KB;
+        ws_ptr[1] = w_s + ((size_t)e * row_blocks + inter / GROUP + rb) * KB;
+    } else {
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) {
+            const int row = rb * 256 + wave * 64 + t * 16;
+            tile_base[t] = w_q + ((size_t)e * n_rows + row) * K;
+        }
+        // wavefronts 0,1 sit in the first 128-row block, 2,3 in the second
+        ws_ptr[0] = w_s + ((size_t)e * row_blocks + rb * 2 + (wave >> 1)) * KB;
+        ws_ptr[1] = ws_ptr[0];
+    }
+
+    // load side: lane j of instruction i fills slot i*64 + j = (row i*8 + j/8, position j%8),
+    // i.e. fetches chunk (j%8) ^ (j/8) of that row
+    const uint32_t ld_row = lane >> 3;
+    const uint32_t ld_chunk = (lane & 7) ^ ld_row;
+    const uint32_t ld_off = ld_row * (uint32_t)K + 16 * ld_chunk;  // + 8*K for the second instruction
+    // read side: lane (col, g) takes chunks g and 4+g of row col
+    const uint32_t rd_off = (col * 8 + (g ^ (col & 7))) * 16;
+
+    const uint32_t ring_base = (uint32_t)(size_t)((lds_void_ptr)s_ring) + wave * (DEPTH * STAGE_BYTES);
+    typedef const __attribute__((address_space(3))) intx4* lds_x4;
+    const __attribute__((address_space(3))) uint8_t* ring_ptr =
+        (const __attribute__((address_space(3))) uint8_t*)s_ring + wave * (DEPTH * STAGE_BYTES);
+
+    for (int pass_begin = begin; pass_begin < end; pass_begin += 16 * NT) {
+        // activation rows: the one this lane loads (row ld_row / ld_row + 8 of tile nt) and the
+        // one whose results it ends up holding (col)
+        const uint8_t* b_ld[NT][2];
+        int pos[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            pos[nt] = pass_begin + 16 * nt + col;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                int p = pass_begin + 16 * nt + i * 8 + (int)ld_row;
+                p = p < end ? p : end - 1;  // clamped rows are computed, not stored
+                const int row = GATE_UP ? sorted_pairs[p] / top_k : p;
+                b_ld[nt][i] = a_q + (size_t)row * K + 16 * ld_chunk;
+            }
+        }
+        __syncthreads();  // the previous pass is done with s_bscale / s_amax
+        for (int i = threadIdx.x; i < KB * NT * 16; i += 256) {
+            const int kb = i / (NT * 16);
+            const int c = i - kb * (NT * 16);
+            int p = pass_begin + c;
+            p = p < end ? p : end - 1;
+            const int row = GATE_UP ? sorted_pairs[p] / top_k : p;
+            s_bscale[kb][c] = a_s[(size_t)row * KB + kb];
+        }
+        __syncthreads();
+        wait_vmcnt<0>();  // nothing of the compiler's is in flight when the counted loads start
+
+        auto issue_stage = [&](int kb) {
+            const uint32_t stage = ring_base + (kb % DEPTH) * STAGE_BYTES;
+#pragma unroll
+            for (int t = 0; t < TILES; ++t) {
+                dma16(tile_base[t] + (size_t)kb * GROUP, ld_off, stage + t * TILE_BYTES);
+                dma16(tile_base[t] + (size_t)kb * GROUP + (size_t)8 * K, ld_off, stage + t * TILE_BYTES + 1024);
+            }
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                dma16_ptr(b_ld[nt][0] + (size_t)kb * GROUP, stage + (TILES + nt) * TILE_BYTES);
+                dma16_ptr(b_ld[nt][1] + (size_t)kb * GROUP, stage + (TILES + nt) * TILE_BYTES + 1024);
+            }
+        };
+
+        floatx4 acc[NT][TILES];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int t = 0; t < TILES; ++t) acc[nt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+        for (int d = 0; d < DEPTH - 1; ++d)
+            if (d < KB) issue_stage(d);
+
+        for (int kb = 0; kb < KB; ++kb) {
+            if (kb + DEPTH - 1 < KB) {
+                issue_stage(kb + DEPTH - 1);
+                wait_vmcnt<(DEPTH - 1) * PER_STAGE>();
+            } else if (kb + DEPTH - 2 < KB && DEPTH > 2) {
+                wait_vmcnt<(DEPTH - 2) * PER_STAGE>();
+            } else {
+                wait_vmcnt<0>();
+            }
+            const __attribute__((address_space(3))) uint8_t* stage = ring_ptr + (kb % DEPTH) * STAGE_BYTES;
+            const float ws0 = ws_ptr[0][kb];
+            const float ws1 = ws_ptr[1][kb];
+            intx8 a[TILES];
+#pragma unroll
+            for (int t = 0; t < TILES; ++t) {
+                const intx4 lo = *(lds_x4)(stage + t * TILE_BYTES + rd_off);
+                const intx4 hi = *(lds_x4)(stage + t * TILE_BYTES + (rd_off ^ 64));
+                a[t] = join(lo, hi);
+            }
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const intx4 lo = *(lds_x4)(stage + (TILES + nt) * TILE_BYTES + rd_off);
+                const intx4 hi = *(lds_x4)(stage + (TILES + nt) * TILE_BYTES + (rd_off ^ 64));
+                const intx8 b = join(lo, hi);
+                const float bs = s_bscale[kb][nt * 16 + col];
+#pragma unroll
+                for (int t = 0; t < TILES; ++t) {
+                    const floatx4 part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                        a[t], b, floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+                    acc[nt][t] += part * (bs * ((t >> 1) ? ws1 : ws0));
+                }
+            }
+            asm volatile("" ::: "memory");  // this stage's LDS reads stay above the next refill
+        }
+
+        if (GATE_UP) {
+            floatx4 h[NT][2];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                float amax = 0.f;
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const float v = silu(acc[nt][i][r]) * acc[nt][2 + i][r];
+                        h[nt][i][r] = v;
+                        amax = fmaxf(amax, fabsf(v));
+                    }
+                }
+                amax = fmaxf(amax, __shfl_xor(amax, 16));
+                amax = fmaxf(amax, __shfl_xor(amax, 32));
+                if (g == 0) s_amax[wave][nt * 16 + col] = amax;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const int idx = nt * 16 + col;
+                const float amax =
+                    fmaxf(fmaxf(s_amax[0][idx], s_amax[1][idx]), fmaxf(s_amax[2][idx], s_amax[3][idx]));
+                const float scale = fmaxf(amax, AMAX_FLOOR) * INV_E4M3_MAX;
+                if (pos[nt] < end) {
+#pragma unroll
+                    for (int i = 0; i < 2; ++i) {
+                        float q[4];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            q[r] = fminf(fmaxf(h[nt][i][r] / scale, -E4M3_MAX), E4M3_MAX);
+                        }
+                        int packed = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], 0, false);
+                        packed = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], packed, true);
+                        *reinterpret_cast<int*>(h_q + (size_t)pos[nt] * inter + rb * GROUP + wave * 32 +
+                                                i * 16 + 4 * g) = packed;
+                    }
+                    if (wave == 0 && g == 0) h_s[(size_t)pos[nt] * (inter / GROUP) + rb] = scale;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                if (pos[nt] < end) {
+#pragma unroll
+                    for (int t = 0; t < TILES; ++t) {
+                        *reinterpret_cast<floatx4*>(y + (size_t)pos[nt] * n_rows + rb * 256 + wave * 64 +
+                                                    t * 16 + 4 * g) = acc[nt][t];
+                    }
+                }
+            }
+        }
+    }
+}
+
 bool check_common(int hidden, int inter, int n_experts) {
     return hidden > 0 && inter > 0 && n_experts > 0 && hidden % GROUP == 0 && inter % GROUP == 0 &&
            n_experts <= 65535;
@@ -206,7 +455,8 @@ bool check_common(int hidden, int inter, int n_experts) {
 // h_q [pairs, inter] e4m3 and h_s [pairs, inter/128] fp32 (rows in sorted order) from
 // x_q [tokens, hidden] e4m3, x_s [tokens, hidden/128], w13_q [E, 2*inter, hidden] e4m3,
 // w13_s [E, 2*inter/128, hidden/128].
-// config: 0 sizes the pass from max_pairs_hint; 1, 2, 4 force 16, 32, 64 pairs per pass.
+// config: 0 sizes the pass from the average pairs per expert; 1, 2, 4 force 16, 32, 64 pairs per
+// pass; adding 8 selects the kernel that loads MFMA operands directly instead of staging in LDS.
 extern "C" void moe_gate_up_launcher(void* h_q, float* h_s, const void* x_q, const float* x_s,
                                      const void* w13_q, const float* w13_s, const int* sorted_pairs,
                                      const int* expert_offsets, int tokens, int hidden, int inter,
@@ -226,21 +476,34 @@ extern "C" void moe_gate_up_launcher(void* h_q, float* h_s, const void* x_q, con
     auto* hq = static_cast<uint8_t*>(h_q);
     const auto* xq = static_cast<const uint8_t*>(x_q);
     const auto* wq = static_cast<const uint8_t*>(w13_q);
-    int nt = config;
+    int nt = config & 7;
     if (nt != 1 && nt != 2 && nt != 4) {
         const long avg = (long)tokens * top_k / n_experts;  // pairs per expert if spread evenly
         nt = avg <= 16 ? 1 : avg <= 32 ? 2 : 4;
     }
+    const bool lds_path = config < 8 && hidden / GROUP <= 64;  // config 8+nt: direct-operand loads
     switch (nt) {
         case 1:
-            moe_stream_gemm_kernel<true, 1><<<grid, 256, 0, stream>>>(
-                wq, w13_s, xq, x_s, sorted_pairs, expert_offsets, hq, h_s, nullptr, hidden, 2 * inter,
-                inter, top_k);
+            if (lds_path) {
+                moe_stream_gemm_lds_kernel<true, 1><<<grid, 256, 0, stream>>>(
+                    wq, w13_s, xq, x_s, sorted_pairs, expert_offsets, hq, h_s, nullptr, hidden,
+                    2 * inter, inter, top_k);
+            } else {
+                moe_stream_gemm_kernel<true, 1><<<grid, 256, 0, stream>>>(
+                    wq, w13_s, xq, x_s, sorted_pairs, expert_offsets, hq, h_s, nullptr, hidden,
+                    2 * inter, inter, top_k);
+            }
             break;
         case 2:
-            moe_stream_gemm_kernel<true, 2><<<grid, 256, 0, stream>>>(
-                wq, w13_s, xq, x_s, sorted_pairs, expert_offsets, hq, h_s, nullptr, hidden, 2 * inter,
-                inter, top_k);
+            if (lds_path) {
+                moe_stream_gemm_lds_kernel<true, 2><<<grid, 256, 0, stream>>>(
+                    wq, w13_s, xq, x_s, sorted_pairs, expert_offsets, hq, h_s, nullptr, hidden,
+                    2 * inter, inter, top_k);
+            } else {
+                moe_stream_gemm_kernel<true, 2><<<grid, 256, 0, stream>>>(
+                    wq, w13_s, xq, x_s, sorted_pairs, expert_offsets, hq, h_s, nullptr, hidden,
+                    2 * inter, inter, top_k);
+            }
             break;
         default:
             moe_stream_gemm_kernel<true, 4><<<grid, 256, 0, stream>>>(
@@ -270,21 +533,35 @@ extern "C" void moe_down_launcher(float* y, const void* h_q, const float* h_s, c
     const dim3 grid(hidden / GROUP, n_experts);
     const auto* hq = static_cast<const uint8_t*>(h_q);
     const auto* wq = static_cast<const uint8_t*>(w2_q);
-    int nt = config;
+    int nt = config & 7;
     if (nt != 1 && nt != 2 && nt != 4) {
         const long avg = (long)tokens * top_k / n_experts;
         nt = avg <= 16 ? 1 : avg <= 32 ? 2 : 4;
     }
+    const bool lds_path = config < 8 && hidden % 256 == 0 && inter / GROUP <= 64;
+    const dim3 grid256(hidden / 256, n_experts);
     switch (nt) {
         case 1:
-            moe_stream_gemm_kernel<false, 1><<<grid, 256, 0, stream>>>(
-                wq, w2_s, hq, h_s, nullptr, expert_offsets, nullptr, nullptr, y, inter, hidden, inter,
-                top_k);
+            if (lds_path) {
+                moe_stream_gemm_lds_kernel<false, 1><<<grid256, 256, 0, stream>>>(
+                    wq, w2_s, hq, h_s, nullptr, expert_offsets, nullptr, nullptr, y, inter, hidden,
+                    inter, top_k);
+            } else {
+                moe_stream_gemm_kernel<false, 1><<<grid, 256, 0, stream>>>(
+                    wq, w2_s, hq, h_s, nullptr, expert_offsets, nullptr, nullptr, y, inter, hidden,
+                    inter, top_k);
+            }
             break;
         case 2:
-            moe_stream_gemm_kernel<false, 2><<<grid, 256, 0, stream>>>(
-                wq, w2_s, hq, h_s, nullptr, expert_offsets, nullptr, nullptr, y, inter, hidden, inter,
-                top_k);
+            if (lds_path) {
+                moe_stream_gemm_lds_kernel<false, 2><<<grid256, 256, 0, stream>>>(
+                    wq, w2_s, hq, h_s, nullptr, expert_offsets, nullptr, nullptr, y, inter, hidden,
+                    inter, top_k);
+            } else {
+                moe_stream_gemm_kernel<false, 2><<<grid, 256, 0, stream>>>(
+                    wq, w2_s, hq, h_s, nullptr, expert_offsets, nullptr, nullptr, y, inter, hidden,
+                    inter, top_k);
+            }
             break;
         default:
             moe_stream_gemm_kernel<false, 4><<<grid, 256, 0, stream>>>(
