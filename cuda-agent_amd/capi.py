@@ -26,6 +26,7 @@ SIGNATURES = {
     'sparse_mla_decode_workspace_bytes': (c_size_t, [c_int, c_int, c_int, c_int]),
     'moe_route_launcher': (None, [_P, _P, _P, c_int, c_int, c_int, c_int, _P]),
     'moe_sort_launcher': (None, [_P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P]),
+    'moe_route_sort_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P]),
     'moe_quant_bf16_launcher': (None, [_P, _P, _P, c_int, c_int, c_int, _P]),
     'moe_gate_up_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int,
                                     c_int, _P]),

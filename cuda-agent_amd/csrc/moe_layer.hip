@@ -10,6 +10,10 @@ extern "C" void moe_route_launcher(int* ids, float* weights, const float* logits
 extern "C" void moe_sort_launcher(int* sorted_pairs, int* pair_pos, int* expert_offsets,
                                   int* chunk_scratch, const int* ids, int tokens, int n_experts,
                                   int top_k, int config, hipStream_t stream);
+extern "C" void moe_route_sort_launcher(int* ids, float* weights, int* sorted_pairs, int* pair_pos,
+                                        int* expert_offsets, int* chunk_scratch, const float* logits,
+                                        int tokens, int n_experts, int top_k, int config,
+                                        hipStream_t stream);
 extern "C" void moe_quant_bf16_launcher(void* q, float* scales, const void* x, int rows, int cols,
                                         int config, hipStream_t stream);
 extern "C" void moe_gate_up_launcher(void* h_q, float* h_s, const void* x_q, const float* x_s,
@@ -28,7 +32,7 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 
 // out[t, :] = sum_k weights[t, k] * y[pair_pos[t*top_k + k], :], k ascending, fp32.
-// One workgroup per token, 4 columns per lane and pass.
+// blockIdx.x is the token, blockIdx.y a 1024-column slice; 4 columns per lane.
 template <typename OUT>
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y,
                                                           const float* __restrict__ weights,
@@ -36,7 +40,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
                                                           OUT* __restrict__ out, int hidden,
                                                           int top_k) {
     const int t = blockIdx.x;
-    for (int c = threadIdx.x * 4; c < hidden; c += 1024) {
+    for (int c = (blockIdx.y * 256 + threadIdx.x) * 4; c < hidden; c += gridDim.y * 1024) {
         floatx4 acc = {0.f, 0.f, 0.f, 0.f};
         for (int k = 0; k < top_k; ++k) {
             const int pos = pair_pos[(size_t)t * top_k + k];
@@ -72,12 +76,13 @@ extern "C" void moe_combine_launcher(void* out, const float* y, const float* wei
         caa::set_status(CAA_BAD_ARGUMENT);
         return;
     }
+    const dim3 grid(tokens, (hidden + 1023) / 1024);
     if (out_dtype == 0) {
-        moe_combine_kernel<__bf16><<<tokens, 256, 0, stream>>>(y, weights, pair_pos,
-                                                              static_cast<__bf16*>(out), hidden, top_k);
+        moe_combine_kernel<__bf16><<<grid, 256, 0, stream>>>(y, weights, pair_pos,
+                                                            static_cast<__bf16*>(out), hidden, top_k);
     } else {
-        moe_combine_kernel<float><<<tokens, 256, 0, stream>>>(y, weights, pair_pos,
-                                                             static_cast<float*>(out), hidden, top_k);
+        moe_combine_kernel<float><<<grid, 256, 0, stream>>>(y, weights, pair_pos,
+                                                           static_cast<float*>(out), hidden, top_k);
     }
 }
 
@@ -123,9 +128,8 @@ extern "C" void moe_fp8_launcher(void* out, const void* x, const float* logits, 
         caa::set_status(CAA_WORKSPACE_TOO_SMALL);
         return;
     }
-    moe_route_launcher(w.ids, w.weights, logits, tokens, n_experts, top_k, 0, stream);
-    moe_sort_launcher(w.sorted_pairs, w.pair_pos, w.expert_offsets, w.chunk_hist, w.ids, tokens,
-                      n_experts, top_k, 0, stream);
+    moe_route_sort_launcher(w.ids, w.weights, w.sorted_pairs, w.pair_pos, w.expert_offsets, w.chunk_hist,
+                            logits, tokens, n_experts, top_k, 0, stream);
     moe_quant_bf16_launcher(w.x_q, w.x_s, x, tokens, hidden, 0, stream);
     moe_gate_up_launcher(w.h_q, w.h_s, w.x_q, w.x_s, w13_q, w13_s, w.sorted_pairs, w.expert_offsets,
                          tokens, hidden, inter, n_experts, top_k, config, stream);

@@ -141,7 +141,92 @@ __global__ __launch_bounds__(256) void moe_scatter_kernel(const int* __restrict_
     }
 }
 
+// Routing and sort of a small batch in one workgroup (tokens*top_k <= 1024 pairs): wavefronts
+// route tokens round-robin, keeping the expert ids in LDS; each pair then finds its position as
+// (first position of its expert) + (number of earlier pairs with the same expert), which is
+// the same stable order the chunked path produces.
+template <int PER_LANE>
+__global__ __launch_bounds__(1024) void moe_route_sort_small_kernel(
+    const float* __restrict__ logits, int* __restrict__ ids, float* __restrict__ weights,
+    int* __restrict__ sorted_pairs, int* __restrict__ pair_pos, int* __restrict__ expert_offsets,
+    int tokens, int n_experts, int top_k) {
+    __shared__ int s_ids[1024];
+    __shared__ int s_count[512 + 1];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int pairs = tokens * top_k;
+    for (int e = threadIdx.x; e <= n_experts; e += 1024) s_count[e] = 0;
+    for (int t = wave; t < tokens; t += 16) {
+        unsigned long long key[PER_LANE];
+#pragma unroll
+        for (int j = 0; j < PER_LANE; ++j) {
+            const int e = j * 64 + lane;
+            key[j] = e < n_experts ? rank_key(logits[(size_t)t * n_experts + e], e) : 0ull;
+        }
+        float my_score = 0.f, total = 0.f;
+        int my_id = 0;
+        for (int k = 0; k < top_k; ++k) {
+            unsigned long long best = 0ull;
+#pragma unroll
+            for (int j = 0; j < PER_LANE; ++j) best = key[j] > best ? key[j] : best;
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) {
+                const unsigned long long other = __shfl_xor(best, off);
+                best = other > best ? other : best;
+            }
+            const int id = 0x7fffffff - (int)(unsigned)(best & 0xffffffffull);
+#pragma unroll
+            for (int j = 0; j < PER_LANE; ++j) {
+                if (j * 64 + lane == id) key[j] = 0ull;
+            }
+            const float score = 1.f / (1.f + expf(-logits[(size_t)t * n_experts + id]));
+            total += score;
+            if (lane == k) {
+                my_score = score;
+                my_id = id;
+            }
+        }
+        if (lane < top_k) {
+            ids[(size_t)t * top_k + lane] = my_id;
+            weights[(size_t)t * top_k + lane] = my_score / total;
+            s_ids[t * top_k + lane] = my_id;
+        }
+    }
+    __syncthreads();
+    const int p = threadIdx.x;
+    int mine = -1, rank = 0;
+    if (p < pairs) {
+        mine = s_ids[p];
+        atomicAdd(&s_count[mine], 1);
+        for (int i = 0; i < p; ++i) rank += s_ids[i] == mine;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {  // exclusive scan of the counts, in place
+        int running = 0;
+        for (int e = 0; e < n_experts; ++e) {
+            const int c = s_count[e];
+            s_count[e] = running;
+            running += c;
+        }
+        s_count[n_experts] = running;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e <= n_experts; e += 1024) expert_offsets[e] = s_count[e];
+    if (p < pairs) {
+        const int pos = s_count[mine] + rank;
+        sorted_pairs[pos] = p;
+        pair_pos[p] = pos;
+    }
+}
+
 }  // namespace
+
+// Routing followed by the sort, in one launch when the batch is small (tokens*top_k <= 1024),
+// otherwise as moe_route_launcher + moe_sort_launcher. Same outputs as those two.
+extern "C" void moe_route_sort_launcher(int* ids, float* weights, int* sorted_pairs, int* pair_pos,
+                                        int* expert_offsets, int* chunk_scratch, const float* logits,
+                                        int tokens, int n_experts, int top_k, int config,
+                                        hipStream_t stream);
 
 // ids [tokens, top_k] int32 and weights [tokens, top_k] fp32 from logits [tokens, n_experts] fp32.
 extern "C" void moe_route_launcher(int* ids, float* weights, const float* logits, int tokens,
@@ -190,4 +275,32 @@ extern "C" void moe_sort_launcher(int* sorted_pairs, int* pair_pos, int* expert_
                                                                  n_experts);
     moe_scatter_kernel<<<chunks, 256, pairs_per_chunk * sizeof(int), stream>>>(
         ids, chunk_scratch, sorted_pairs, pair_pos, pairs, pairs_per_chunk, n_experts);
+}
+
+extern "C" void moe_route_sort_launcher(int* ids, float* weights, int* sorted_pairs, int* pair_pos,
+                                        int* expert_offsets, int* chunk_scratch, const float* logits,
+                                        int tokens, int n_experts, int top_k, int config,
+                                        hipStream_t stream) {
+    if (tokens <= 0) return;
+    if (n_experts <= 0 || n_experts > 512 || top_k <= 0 || top_k > 64 || top_k > n_experts) {
+        caa::set_status(CAA_UNSUPPORTED_SHAPE);
+        return;
+    }
+    if (!ids || !weights || !sorted_pairs || !pair_pos || !expert_offsets || !chunk_scratch || !logits) {
+        caa::set_status(CAA_BAD_ARGUMENT);
+        return;
+    }
+    if ((long)tokens * top_k <= 1024 && config != 1) {
+        if (n_experts <= 256) {
+            moe_route_sort_small_kernel<4><<<1, 1024, 0, stream>>>(
+                logits, ids, weights, sorted_pairs, pair_pos, expert_offsets, tokens, n_experts, top_k);
+        } else {
+            moe_route_sort_small_kernel<8><<<1, 1024, 0, stream>>>(
+                logits, ids, weights, sorted_pairs, pair_pos, expert_offsets, tokens, n_experts, top_k);
+        }
+        return;
+    }
+    moe_route_launcher(ids, weights, logits, tokens, n_experts, top_k, 0, stream);
+    moe_sort_launcher(sorted_pairs, pair_pos, expert_offsets, chunk_scratch, ids, tokens, n_experts,
+                      top_k, 0, stream);
 }

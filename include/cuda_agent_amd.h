@@ -119,6 +119,12 @@ void moe_sort_launcher(int* sorted_pairs, int* pair_pos, int* expert_offsets, in
                        const int* ids, int tokens, int n_experts, int top_k, int config,
                        hipStream_t stream);
 
+/* moe_route_launcher followed by moe_sort_launcher, as one kernel when tokens*top_k <= 1024 (the
+ * decode case); same outputs. config 1 forces the two-step path. */
+void moe_route_sort_launcher(int* ids, float* weights, int* sorted_pairs, int* pair_pos,
+                             int* expert_offsets, int* chunk_scratch, const float* logits, int tokens,
+                             int n_experts, int top_k, int config, hipStream_t stream);
+
 /* q [rows, cols] e4m3 codes and scales [rows, cols/128] fp32 from x [rows, cols] bf16. */
 void moe_quant_bf16_launcher(void* q, float* scales, const void* x, int rows, int cols, int config,
                              hipStream_t stream);
