@@ -27,6 +27,10 @@ struct Workspace {
     uint8_t* h_q;         // [T*k*I] e4m3 silu(g)*u, rows in sorted order
     float* h_s;           // [T*k*I/128]
     float* y;             // [T*k*H] expert outputs, rows in sorted order
+    int* tile_start;      // [E+1]  first 256-pair tile of every expert (tiled path)
+    float* xs_t;          // [H/128][scale_stride] activation scales by sorted position, transposed
+    float* hs_t;          // [I/128][scale_stride] the same for h
+    int scale_stride;     // pairs rounded up to 256, plus 256 of padding
     size_t bytes;
 };
 
@@ -55,6 +59,10 @@ inline Workspace carve_workspace(void* base, int tokens, int hidden, int inter, 
     w.h_q = reinterpret_cast<uint8_t*>(take(pairs * inter));
     w.h_s = reinterpret_cast<float*>(take(pairs * (inter / GROUP) * 4));
     w.y = reinterpret_cast<float*>(take(pairs * hidden * 4));
+    w.scale_stride = (int)(align_up(pairs, 256) + 256);
+    w.tile_start = reinterpret_cast<int*>(take(((size_t)n_experts + 1) * 4));
+    w.xs_t = reinterpret_cast<float*>(take((size_t)(hidden / GROUP) * w.scale_stride * 4));
+    w.hs_t = reinterpret_cast<float*>(take((size_t)(inter / GROUP) * w.scale_stride * 4));
     w.bytes = off;
     return w;
 }

@@ -1,0 +1,346 @@
+// Grouped FP8 GEMMs of the MoE layer, LDS-tiled form (many pairs per expert: prefill).
+//
+// A workgroup of 8 wavefronts computes a 256 (weight rows) x 256 (pairs) tile of one expert:
+// per 128-block of K it brings 32 KB of weights, 32 KB of activations and the 256 activation
+// scales of the block into LDS with global->LDS loads in which 8 lanes fetch one full 128-byte
+// line of a row (two stages: the next block loads while the current one is multiplied), and
+// each wavefront multiplies a 64-row x 128-pair slice on v_mfma_f32_32x32x64_f8f6f4:
+//
+//   weights are the A operand (rows -> M), activations the B operand (pairs -> N), so that in the
+//   result layout a lane holds 16 weight rows of ONE pair and the block's scale product
+//   x_s[pair, kb] * w_s[row block, kb] is a per-lane scalar;
+//   the unscaled partial of one 128-block (two MFMAs of K = 64) is folded into the fp32
+//   accumulator with one multiply-add per value (the block scales are arbitrary fp32 and vary
+//   along K, so they can be applied neither once at the end nor by the hardware's
+//   power-of-two block scaling);
+//   the two A tiles of a wavefront stay in registers for the whole block while the four B
+//   tiles stream through: 24 KB of LDS reads per wavefront and block, 16 MFMAs.
+//
+// LDS slot of 16-byte chunk c of row r: r*8 + (c ^ (r & 7)), conflict-free for the fill and
+// for both operand reads. For gate/up the 256 rows are 128 gate rows and the matching 128 up
+// rows, each wavefront holding 32 of either, so SiLU(gate)*up and the e4m3 requantisation of
+// the 128-column group happen in the epilogue without leaving the workgroup.
+#include "launch_status.hpp"
+#include "moe_common.hpp"
+
+namespace {
+
+using namespace moe;
+
+typedef int intx8 __attribute__((ext_vector_type(8)));
+typedef int intx4 __attribute__((ext_vector_type(4)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+typedef const __attribute__((address_space(3))) uint8_t* lds_bytes;
+typedef const __attribute__((address_space(3))) intx4* lds_x4;
+
+constexpr int TILE_PAIRS = 256;
+constexpr int TILE_ROWS = 256;
+constexpr int STAGE_A = TILE_ROWS * GROUP;    // 32 KB
+constexpr int STAGE_B = TILE_PAIRS * GROUP;   // 32 KB
+constexpr int STAGE_S = TILE_PAIRS * 4;       // 1 KB of scales
+constexpr int STAGE_BYTES = STAGE_A + STAGE_B + STAGE_S;
+
+__device__ __forceinline__ intx8 join(intx4 lo, intx4 hi) {
+    return intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+}
+
+__device__ __forceinline__ float silu(float x) { return x / (1.f + expf(-x)); }
+
+__device__ __forceinline__ void wait_all_loads() {
+    __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));  // vmcnt(0)
+    asm volatile("" ::: "memory");
+}
+
+// 64 lanes x 16 bytes, global -> LDS (lds_base + lane*16); asm so that the compiler does not
+// make every later LDS read wait for it: completion is awaited once per block, before the barrier.
+__device__ __forceinline__ void dma16(const void* base, uint32_t lane_byte_offset, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(lane_byte_offset), "s"(base), "s"(lds_base)
+                 : "memory", "m0");
+}
+__device__ __forceinline__ void dma16_ptr(const void* lane_ptr, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(lane_ptr), "s"(lds_base)
+                 : "memory", "m0");
+}
+
+// tile_start[e] = number of 256-pair tiles of the experts before e (tile_start[E] = total).
+__global__ __launch_bounds__(1024) void moe_tile_start_kernel(const int* __restrict__ expert_offsets,
+                                                              int* __restrict__ tile_start,
+                                                              int n_experts) {
+    if (threadIdx.x == 0) {
+        int running = 0;
+        for (int e = 0; e < n_experts; ++e) {
+            tile_start[e] = running;
+            running += (expert_offsets[e + 1] - expert_offsets[e] + TILE_PAIRS - 1) / TILE_PAIRS;
+        }
+        tile_start[n_experts] = running;
+    }
+}
+
+// xs_t[kb][pos] = x_s[token of sorted position pos][kb]
+__global__ __launch_bounds__(256) void moe_gather_scales_kernel(const float* __restrict__ x_s,
+                                                                const int* __restrict__ sorted_pairs,
+                                                                float* __restrict__ xs_t, int pairs,
+                                                                int stride, int kb_count, int top_k) {
+    const int pos = blockIdx.x * 256 + threadIdx.x;
+    if (pos >= pairs) return;
+    const int token = sorted_pairs[pos] / top_k;
+    for (int kb = 0; kb < kb_count; ++kb) {
+        xs_t[(size_t)kb * stride + pos] = x_s[(size_t)token * kb_count + kb];
+    }
+}
+
+// grid: x = row tile, y = pair tile (over all experts, see tile_start)
+template <bool GATE_UP>
+__global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
+    const uint8_t* __restrict__ w_q, const float* __restrict__ w_s, const uint8_t* __restrict__ a_q,
+    const float* __restrict__ as_t, const int* __restrict__ sorted_pairs,
+    const int* __restrict__ expert_offsets, const int* __restrict__ tile_start,
+    uint8_t* __restrict__ h_q, float* __restrict__ h_s, float* __restrict__ hs_t, float* __restrict__ y,
+    int K, int n_rows, int inter, int top_k, int n_experts, int scale_stride) {
+    __shared__ __attribute__((aligned(16))) uint8_t s_stage[2 * STAGE_BYTES];
+
+    // which expert and which 256-pair tile of it
+    const int total_tiles = tile_start[n_experts];
+    if ((int)blockIdx.y >= total_tiles) return;
+    int lo = 0, hi = n_experts;  // largest e with tile_start[e] <= blockIdx.y
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (tile_start[mid] <= (int)blockIdx.y) lo = mid; else hi = mid;
+    }
+    const int e = lo;
+    const int begin = expert_offsets[e] + ((int)blockIdx.y - tile_start[e]) * TILE_PAIRS;
+    int cnt = expert_offsets[e + 1] - begin;
+    cnt = cnt > TILE_PAIRS ? TILE_PAIRS : cnt;
+    const int rb = blockIdx.x;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int rg = wave & 3;   // 64-row group (gate/up: 32 gate + 32 up rows)
+    const int th = wave >> 2;  // 128-pair half
+    const int KB = K / GROUP;
+    const int row_blocks = n_rows / GROUP;
+    const int r32 = lane & 31;
+    const int half = lane >> 5;
+
+    // ---- fill side -------------------------------------------------------------------------
+    // instruction j of a region covers its rows 8j..8j+7; lane -> row 8j + lane/8, chunk
+    // (lane%8) ^ (lane/8). This wavefront issues instructions 4*wave .. 4*wave+3 of A and of B.
+    const uint32_t ld_row = lane >> 3;
+    const uint32_t ld_chunk = (lane & 7) ^ ld_row;
+    const uint32_t ld_off = ld_row * (uint32_t)K + 16 * ld_chunk;
+    const uint8_t* a_src[4];
+    const uint8_t* b_src[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int ar = (4 * wave + i) * 8;  // first of the 8 tile rows of this instruction
+        int row;
+        if (GATE_UP) row = (ar < 128 ? 0 : inter - 128) + rb * GROUP + ar;
+        else row = rb * TILE_ROWS + ar;
+        a_src[i] = w_q + ((size_t)e * n_rows + row) * K;
+        int p = (4 * wave + i) * 8 + (int)ld_row;
+        p = begin + (p < cnt ? p : cnt - 1);  // rows past the tile's end repeat the last one
+        const int arow = GATE_UP ? sorted_pairs[p] / top_k : p;
+        b_src[i] = a_q + (size_t)arow * K + 16 * ld_chunk;
+    }
+    const float* s_src = as_t + begin;  // + kb*scale_stride; 256 floats, the tail is padding
+    const float* ws0;
+    const float* ws1;
+    if (GATE_UP) {
+        ws0 = w_s + ((size_t)e * row_blocks + rb) * KB;
+        ws1 = w_s + ((size_t)e * row_blocks + inter / GROUP + rb) * KB;
+    } else {
+        ws0 = w_s + ((size_t)e * row_blocks + rb * 2 + (rg >> 1)) * KB;
+        ws1 = ws0;
+    }
+
+    const uint32_t stage_base = (uint32_t)(size_t)((lds_void_ptr)s_stage);
+    auto issue_stage = [&](int kb) {
+        const uint32_t st = stage_base + (kb & 1) * STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            dma16(a_src[i] + (size_t)kb * GROUP, ld_off, st + (4 * wave + i) * 1024);
+            dma16_ptr(b_src[i] + (size_t)kb * GROUP, st + STAGE_A + (4 * wave + i) * 1024);
+        }
+        if (wave == 0) {
+            dma16(s_src + (size_t)kb * scale_stride, lane * 16, st + STAGE_A + STAGE_B);
+        }
+    };
+
+    // ---- read side -------------------------------------------------------------------------
+    // operand of k-step s, 16-byte piece j: chunk 4s + 2*half + j of row r32 (+32*tile)
+    const uint32_t rd = (r32 * 8 + ((2 * half) ^ (r32 & 7))) * 16;
+    const uint32_t a_row0 = GATE_UP ? rg * 32 : rg * 64;        // A tile 0 of this wavefront
+    const uint32_t a_row1 = GATE_UP ? 128 + rg * 32 : rg * 64 + 32;
+    const lds_bytes stage_ptr = (lds_bytes)s_stage;
+
+    int active_b = (cnt - th * 128 + 31) / 32;  // B tiles of this wavefront that hold pairs
+    active_b = active_b < 0 ? 0 : active_b > 4 ? 4 : active_b;
+
+    floatx16 acc[2][4];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) acc[a][b] = floatx16{0};
+
+    issue_stage(0);
+    for (int kb = 0; kb < KB; ++kb) {
+        wait_all_loads();
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (kb + 1 < KB) issue_stage(kb + 1);
+
+        const lds_bytes st = stage_ptr + (kb & 1) * STAGE_BYTES;
+        const float w0 = ws0[kb];
+        const float w1 = ws1[kb];
+        intx8 A[2][2];  // [tile][k-step]
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            A[0][s] = join(*(lds_x4)(st + a_row0 * GROUP + (rd ^ (64 * s))),
+                           *(lds_x4)(st + a_row0 * GROUP + (rd ^ (64 * s) ^ 16)));
+            A[1][s] = join(*(lds_x4)(st + a_row1 * GROUP + (rd ^ (64 * s))),
+                           *(lds_x4)(st + a_row1 * GROUP + (rd ^ (64 * s) ^ 16)));
+        }
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            if (b < active_b) {
+                const lds_bytes bt = st + STAGE_A + (th * 128 + b * 32) * GROUP;
+                const intx8 B0 = join(*(lds_x4)(bt + rd), *(lds_x4)(bt + (rd ^ 16)));
+                const intx8 B1 = join(*(lds_x4)(bt + (rd ^ 64)), *(lds_x4)(bt + (rd ^ 64 ^ 16)));
+                const float bs = *(const __attribute__((address_space(3))) float*)(
+                    st + STAGE_A + STAGE_B + (th * 128 + b * 32 + r32) * 4);
+                floatx16 p0 = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(A[0][0], B0, floatx16{0}, 0, 0,
+                                                                               0, 0, 0, 0);
+                floatx16 p1 = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(A[1][0], B0, floatx16{0}, 0, 0,
+                                                                               0, 0, 0, 0);
+                p0 = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(A[0][1], B1, p0, 0, 0, 0, 0, 0, 0);
+                p1 = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(A[1][1], B1, p1, 0, 0, 0, 0, 0, 0);
+                acc[0][b] += p0 * (bs * w0);
+                acc[1][b] += p1 * (bs * w1);
+            }
+        }
+        asm volatile("" ::: "memory");
+    }
+    __syncthreads();  // the stages are free: reuse them for the epilogue exchange
+
+    // result layout: register i of acc[a][b] is row 8*(i/4) + 4*half + i%4 of A tile a, pair
+    // th*128 + b*32 + r32 of the tile
+    if (GATE_UP) {
+        float* s_amax = reinterpret_cast<float*>(s_stage);  // [4 row groups][256 pairs]
+        float amax[4];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            float m = 0.f;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const float v = silu(acc[0][b][i]) * acc[1][b][i];
+                acc[0][b][i] = v;
+                m = fmaxf(m, fabsf(v));
+            }
+            m = fmaxf(m, __shfl_xor(m, 32));
+            amax[b] = m;
+            if (half == 0) s_amax[rg * TILE_PAIRS + th * 128 + b * 32 + r32] = m;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int pl = th * 128 + b * 32 + r32;
+            if (pl < cnt) {
+                const float m = fmaxf(fmaxf(s_amax[pl], s_amax[TILE_PAIRS + pl]),
+                                      fmaxf(s_amax[2 * TILE_PAIRS + pl], s_amax[3 * TILE_PAIRS + pl]));
+                const float scale = fmaxf(m, AMAX_FLOOR) * INV_E4M3_MAX;
+                const size_t pos = (size_t)begin + pl;
+#pragma unroll
+                for (int qd = 0; qd < 4; ++qd) {
+                    float q[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        q[r] = fminf(fmaxf(acc[0][b][4 * qd + r] / scale, -E4M3_MAX), E4M3_MAX);
+                    }
+                    int packed = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], 0, false);
+                    packed = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], packed, true);
+                    *reinterpret_cast<int*>(h_q + pos * inter + rb * GROUP + rg * 32 + 8 * qd + 4 * half) =
+                        packed;
+                }
+                if (rg == 0 && half == 0) {
+                    h_s[pos * (inter / GROUP) + rb] = scale;
+                    hs_t[(size_t)rb * scale_stride + pos] = scale;
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int pl = th * 128 + b * 32 + r32;
+            if (pl < cnt) {
+                float* dst = y + ((size_t)begin + pl) * n_rows + rb * TILE_ROWS + rg * 64 + 4 * half;
+#pragma unroll
+                for (int a = 0; a < 2; ++a) {
+#pragma unroll
+                    for (int qd = 0; qd < 4; ++qd) {
+                        *reinterpret_cast<floatx4*>(dst + a * 32 + 8 * qd) =
+                            floatx4{acc[a][b][4 * qd], acc[a][b][4 * qd + 1], acc[a][b][4 * qd + 2],
+                                    acc[a][b][4 * qd + 3]};
+                    }
+                }
+            }
+        }
+    }
+}
+
+}  // namespace
+
+// Scratch the tiled path needs beyond the layer's common workspace:
+//   tile_start [n_experts+1] ints; xs_t [hidden/128][stride] and hs_t [inter/128][stride] floats
+//   with stride = pairs rounded up to 256, plus 256.
+extern "C" void moe_tiled_prepare_launcher(int* tile_start, float* xs_t, const float* x_s,
+                                           const int* sorted_pairs, const int* expert_offsets,
+                                           int tokens, int hidden, int n_experts, int top_k,
+                                           int scale_stride, hipStream_t stream) {
+    if (tokens <= 0) return;
+    const int pairs = tokens * top_k;
+    moe_tile_start_kernel<<<1, 1024, 0, stream>>>(expert_offsets, tile_start, n_experts);
+    moe_gather_scales_kernel<<<(pairs + 255) / 256, 256, 0, stream>>>(x_s, sorted_pairs, xs_t, pairs,
+                                                                    scale_stride, hidden / GROUP, top_k);
+}
+
+extern "C" void moe_gate_up_tiled_launcher(void* h_q, float* h_s, float* hs_t, const void* x_q,
+                                           const float* xs_t, const void* w13_q, const float* w13_s,
+                                           const int* sorted_pairs, const int* expert_offsets,
+                                           const int* tile_start, int tokens, int hidden, int inter,
+                                           int n_experts, int top_k, int scale_stride,
+                                           hipStream_t stream) {
+    if (tokens <= 0) return;
+    if (hidden % GROUP != 0 || inter % GROUP != 0 || hidden <= 0 || inter <= 0) {
+        caa::set_status(CAA_UNSUPPORTED_SHAPE);
+        return;
+    }
+    const int max_tiles = (tokens * top_k) / TILE_PAIRS + n_experts;
+    const dim3 grid(inter / GROUP, max_tiles);
+    moe_tiled_gemm_kernel<true><<<grid, 512, 0, stream>>>(
+        static_cast<const uint8_t*>(w13_q), w13_s, static_cast<const uint8_t*>(x_q), xs_t, sorted_pairs,
+        expert_offsets, tile_start, static_cast<uint8_t*>(h_q), h_s, hs_t, nullptr, hidden, 2 * inter,
+        inter, top_k, n_experts, scale_stride);
+}
+
+extern "C" void moe_down_tiled_launcher(float* y, const void* h_q, const float* hs_t, const void* w2_q,
+                                        const float* w2_s, const int* expert_offsets,
+                                        const int* tile_start, int tokens, int hidden, int inter,
+                                        int n_experts, int top_k, int scale_stride, hipStream_t stream) {
+    if (tokens <= 0) return;
+    if (hidden % TILE_ROWS != 0 || inter % GROUP != 0 || hidden <= 0 || inter <= 0) {
+        caa::set_status(CAA_UNSUPPORTED_SHAPE);
+        return;
+    }
+    const int max_tiles = (tokens * top_k) / TILE_PAIRS + n_experts;
+    const dim3 grid(hidden / TILE_ROWS, max_tiles);
+    moe_tiled_gemm_kernel<false><<<grid, 512, 0, stream>>>(
+        static_cast<const uint8_t*>(w2_q), w2_s, static_cast<const uint8_t*>(h_q), hs_t, nullptr,
+        expert_offsets, tile_start, nullptr, nullptr, nullptr, y, inter, hidden, inter, top_k,
+        n_experts, scale_stride);
+}

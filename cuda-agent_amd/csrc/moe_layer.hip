@@ -24,6 +24,21 @@ extern "C" void moe_down_launcher(float* y, const void* h_q, const float* h_s, c
                                   const float* w2_s, const int* expert_offsets, int tokens, int hidden,
                                   int inter, int n_experts, int top_k, int config, hipStream_t stream);
 
+extern "C" void moe_tiled_prepare_launcher(int* tile_start, float* xs_t, const float* x_s,
+                                           const int* sorted_pairs, const int* expert_offsets,
+                                           int tokens, int hidden, int n_experts, int top_k,
+                                           int scale_stride, hipStream_t stream);
+extern "C" void moe_gate_up_tiled_launcher(void* h_q, float* h_s, float* hs_t, const void* x_q,
+                                           const float* xs_t, const void* w13_q, const float* w13_s,
+                                           const int* sorted_pairs, const int* expert_offsets,
+                                           const int* tile_start, int tokens, int hidden, int inter,
+                                           int n_experts, int top_k, int scale_stride,
+                                           hipStream_t stream);
+extern "C" void moe_down_tiled_launcher(float* y, const void* h_q, const float* hs_t, const void* w2_q,
+                                        const float* w2_s, const int* expert_offsets,
+                                        const int* tile_start, int tokens, int hidden, int inter,
+                                        int n_experts, int top_k, int scale_stride, hipStream_t stream);
+
 namespace {
 
 using namespace moe;
@@ -105,7 +120,8 @@ extern "C" void moe_fp8_workspace_layout(size_t* offsets10, int tokens, int hidd
 }
 
 // The whole layer. out [tokens, hidden] bf16 (out_dtype 0) or fp32 (out_dtype 1).
-// config: 0 = defaults; 1, 2, 4 force 16, 32, 64 pairs per pass of the grouped GEMMs.
+// config: 0 = choose by the average number of pairs per expert (above 32: LDS-tiled GEMMs, else
+// weight streaming); 16 forces the tiled GEMMs; 1, 2, 4 (+8) force streaming, see moe_gate_up_launcher.
 extern "C" void moe_fp8_launcher(void* out, const void* x, const float* logits, const void* w13_q,
                                  const float* w13_s, const void* w2_q, const float* w2_s,
                                  void* workspace, size_t workspace_bytes, int tokens, int hidden,
@@ -131,9 +147,22 @@ extern "C" void moe_fp8_launcher(void* out, const void* x, const float* logits, 
     moe_route_sort_launcher(w.ids, w.weights, w.sorted_pairs, w.pair_pos, w.expert_offsets, w.chunk_hist,
                             logits, tokens, n_experts, top_k, 0, stream);
     moe_quant_bf16_launcher(w.x_q, w.x_s, x, tokens, hidden, 0, stream);
-    moe_gate_up_launcher(w.h_q, w.h_s, w.x_q, w.x_s, w13_q, w13_s, w.sorted_pairs, w.expert_offsets,
-                         tokens, hidden, inter, n_experts, top_k, config, stream);
-    moe_down_launcher(w.y, w.h_q, w.h_s, w2_q, w2_s, w.expert_offsets, tokens, hidden, inter,
-                      n_experts, top_k, config, stream);
+    // Many pairs per expert: LDS-tiled GEMMs (256 x 256 tiles). Few: the weight-streaming form.
+    const bool tiled = config == 16 || (config == 0 && (long)tokens * top_k > 32L * n_experts &&
+                                        hidden % 256 == 0);
+    if (tiled) {
+        moe_tiled_prepare_launcher(w.tile_start, w.xs_t, w.x_s, w.sorted_pairs, w.expert_offsets, tokens,
+                                   hidden, n_experts, top_k, w.scale_stride, stream);
+        moe_gate_up_tiled_launcher(w.h_q, w.h_s, w.hs_t, w.x_q, w.xs_t, w13_q, w13_s, w.sorted_pairs,
+                                   w.expert_offsets, w.tile_start, tokens, hidden, inter, n_experts,
+                                   top_k, w.scale_stride, stream);
+        moe_down_tiled_launcher(w.y, w.h_q, w.hs_t, w2_q, w2_s, w.expert_offsets, w.tile_start, tokens,
+                                hidden, inter, n_experts, top_k, w.scale_stride, stream);
+    } else {
+        moe_gate_up_launcher(w.h_q, w.h_s, w.x_q, w.x_s, w13_q, w13_s, w.sorted_pairs, w.expert_offsets,
+                             tokens, hidden, inter, n_experts, top_k, config, stream);
+        moe_down_launcher(w.y, w.h_q, w.h_s, w2_q, w2_s, w.expert_offsets, tokens, hidden, inter,
+                          n_experts, top_k, config, stream);
+    }
     moe_combine_launcher(out, w.y, w.weights, w.pair_pos, tokens, hidden, top_k, out_dtype, 0, stream);
 }

@@ -161,7 +161,10 @@ void moe_fp8_workspace_layout(size_t* offsets10, int tokens, int hidden, int int
 /* The whole layer: out [tokens, hidden] (bf16 if out_dtype == 0, the operator's output type;
  * fp32 if 1, the same values before the final rounding) from x [tokens, hidden] bf16 and
  * logits [tokens, n_experts] fp32. workspace: moe_fp8_workspace_bytes(...) bytes, 256-byte
- * aligned. hidden and inter multiples of 128. config as for moe_gate_up_launcher. */
+ * aligned. hidden and inter multiples of 128. config: 0 picks the GEMM form from the average number
+ * of pairs per expert (above 32 and hidden % 256 == 0: LDS-tiled 256x256 GEMMs; otherwise the
+ * weight-streaming form); 16 forces the tiled form; 1, 2, 4 (+8) force streaming as for
+ * moe_gate_up_launcher. */
 void moe_fp8_launcher(void* out, const void* x, const float* logits, const void* w13_q,
                       const float* w13_s, const void* w2_q, const float* w2_s, void* workspace,
                       size_t workspace_bytes, int tokens, int hidden, int inter, int n_experts,

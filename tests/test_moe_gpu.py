@@ -163,6 +163,25 @@ def test_layer_small(capi, dev, config):
     check_layer(capi, dev, T=40, H=512, I=256, E=8, k=2, seed=41, config=config)
 
 
+@pytest.mark.parametrize('shape', [(300, 512, 256, 4, 2), (700, 256, 128, 2, 1), (520, 768, 384, 3, 3),
+                                   (64, 256, 128, 4, 4)])
+def test_layer_tiled_gemms(capi, dev, shape):
+    # config 16 forces the LDS-tiled GEMMs: full 256-pair tiles, ragged last tiles, experts with
+    # fewer pairs than one tile, several row tiles
+    T, H, I, E, k = shape
+    check_layer(capi, dev, T=T, H=H, I=I, E=E, k=k, seed=50 + T, config=16)
+
+
+def test_tiled_path_is_chosen_for_many_pairs_per_expert(capi, dev):
+    # 1200 pairs over 8 experts: config 0 takes the tiled form; it must agree with streaming
+    x, logits, w, dts = make_case(dev, 600, 512, 256, 8, 61)
+    a, _ = run_layer(capi, dts, 2, 0, torch.float32)
+    b, _ = run_layer(capi, dts, 2, 4, torch.float32)
+    c, _ = run_layer(capi, dts, 2, 16, torch.float32)
+    assert torch.equal(a, c)
+    assert moe.rel_rms_error(a.cpu(), b.cpu()) <= TOL
+
+
 def test_layer_ragged_expert_load(capi, dev):
     # 3 tokens over 16 experts (most experts empty), then 130 tokens over 4 experts (several
     # passes per expert with a ragged last pass)
