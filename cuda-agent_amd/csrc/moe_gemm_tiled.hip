@@ -41,6 +41,13 @@ constexpr int STAGE_A = TILE_ROWS * GROUP;    // 32 KB
 constexpr int STAGE_B = TILE_PAIRS * GROUP;   // 32 KB
 constexpr int STAGE_S = TILE_PAIRS * 4;       // 1 KB of scales
 constexpr int STAGE_BYTES = STAGE_A + STAGE_B + STAGE_S;
+constexpr int SUPER_ROWS = 4;   // row tiles and pair tiles of the block of workgroups that
+constexpr int SUPER_PAIRS = 8;  // share one XCD's L2
+
+inline int tiled_grid(int row_tiles, int max_pair_tiles) {
+    const int supers = ((row_tiles + SUPER_ROWS - 1) / SUPER_ROWS) * ((max_pair_tiles + SUPER_PAIRS - 1) / SUPER_PAIRS);
+    return ((supers + 7) / 8) * 8 * SUPER_ROWS * SUPER_PAIRS;
+}
 
 __device__ __forceinline__ intx8 join(intx4 lo, intx4 hi) {
     return intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
@@ -95,7 +102,7 @@ __global__ __launch_bounds__(256) void moe_gather_scales_kernel(const float* __r
     }
 }
 
-// grid: x = row tile, y = pair tile (over all experts, see tile_start)
+// grid: 1-D, see the mapping at the top of the kernel
 template <bool GATE_UP>
 __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
     const uint8_t* __restrict__ w_q, const float* __restrict__ w_s, const uint8_t* __restrict__ a_q,
@@ -105,19 +112,28 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
     int K, int n_rows, int inter, int top_k, int n_experts, int scale_stride) {
     __shared__ __attribute__((aligned(16))) uint8_t s_stage[2 * STAGE_BYTES];
 
-    // which expert and which 256-pair tile of it
+    // Workgroup -> (row tile, pair tile). Consecutive workgroup ids go round-robin to the 8 XCDs,
+    // each with its own L2, so the 32 workgroups that run together on one XCD are given a
+    // 4 x 8 block of (row tile, pair tile): they share 4 weight tiles and 8 activation tiles
+    // through that L2 instead of pulling 18 different ones.
     const int total_tiles = tile_start[n_experts];
-    if ((int)blockIdx.y >= total_tiles) return;
-    int lo = 0, hi = n_experts;  // largest e with tile_start[e] <= blockIdx.y
+    const int row_tiles = GATE_UP ? inter / GROUP : n_rows / TILE_ROWS;
+    const int row_blocks4 = (row_tiles + SUPER_ROWS - 1) / SUPER_ROWS;
+    const int linear = blockIdx.x;
+    const int super = ((linear >> 3) / (SUPER_ROWS * SUPER_PAIRS)) * 8 + (linear & 7);
+    const int within = (linear >> 3) % (SUPER_ROWS * SUPER_PAIRS);
+    const int rb = (super % row_blocks4) * SUPER_ROWS + within % SUPER_ROWS;
+    const int pt = (super / row_blocks4) * SUPER_PAIRS + within / SUPER_ROWS;
+    if (rb >= row_tiles || pt >= total_tiles) return;
+    int lo = 0, hi = n_experts;  // largest e with tile_start[e] <= pt
     while (hi - lo > 1) {
         const int mid = (lo + hi) >> 1;
-        if (tile_start[mid] <= (int)blockIdx.y) lo = mid; else hi = mid;
+        if (tile_start[mid] <= pt) lo = mid; else hi = mid;
     }
     const int e = lo;
-    const int begin = expert_offsets[e] + ((int)blockIdx.y - tile_start[e]) * TILE_PAIRS;
+    const int begin = expert_offsets[e] + (pt - tile_start[e]) * TILE_PAIRS;
     int cnt = expert_offsets[e + 1] - begin;
     cnt = cnt > TILE_PAIRS ? TILE_PAIRS : cnt;
-    const int rb = blockIdx.x;
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -321,7 +337,7 @@ extern "C" void moe_gate_up_tiled_launcher(void* h_q, float* h_s, float* hs_t, c
         return;
     }
     const int max_tiles = (tokens * top_k) / TILE_PAIRS + n_experts;
-    const dim3 grid(inter / GROUP, max_tiles);
+    const dim3 grid(tiled_grid(inter / GROUP, max_tiles));
     moe_tiled_gemm_kernel<true><<<grid, 512, 0, stream>>>(
         static_cast<const uint8_t*>(w13_q), w13_s, static_cast<const uint8_t*>(x_q), xs_t, sorted_pairs,
         expert_offsets, tile_start, static_cast<uint8_t*>(h_q), h_s, hs_t, nullptr, hidden, 2 * inter,
@@ -338,7 +354,7 @@ extern "C" void moe_down_tiled_launcher(float* y, const void* h_q, const float* 
         return;
     }
     const int max_tiles = (tokens * top_k) / TILE_PAIRS + n_experts;
-    const dim3 grid(hidden / TILE_ROWS, max_tiles);
+    const dim3 grid(tiled_grid(hidden / TILE_ROWS, max_tiles));
     moe_tiled_gemm_kernel<false><<<grid, 512, 0, stream>>>(
         static_cast<const uint8_t*>(w2_q), w2_s, static_cast<const uint8_t*>(h_q), hs_t, nullptr,
         expert_offsets, tile_start, nullptr, nullptr, nullptr, y, inter, hidden, inter, top_k,
