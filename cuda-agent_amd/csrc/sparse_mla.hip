@@ -296,6 +296,12 @@ __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
+// all of this wavefront's vector-memory AND LDS operations have completed (tiles with padding
+// rows are completed by ordinary LDS stores of zeros, which the other wavefronts read)
+__device__ __forceinline__ void wait_all_memory() {
+    __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (0 << 8));
+}
+
 // grid: x = split, y = request, z = head group of 32*NW heads
 template <int NW>
 __global__ __launch_bounds__(64 * NW) void sparse_mla_split_kernel(
@@ -380,7 +386,7 @@ __global__ __launch_bounds__(64 * NW) void sparse_mla_split_kernel(
         if ((T) + 1 < n_tiles && (T) + 1 < first_masked_tile)                                   \
             wait_vmcnt<PER_WAVE>();                                                             \
         else                                                                                    \
-            wait_vmcnt<0>();                                                                    \
+            wait_all_memory();                                                                  \
         __builtin_amdgcn_s_barrier();                                                           \
         asm volatile("" ::: "memory");                                                          \
         const bool more = (T) + 2 < n_tiles;                                                    \
@@ -432,6 +438,302 @@ __global__ __launch_bounds__(64 * NW) void sparse_mla_split_kernel(
             const int r = 2 * it + half;
             const floatx4 v = *reinterpret_cast<const floatx4*>(stage + r * STAGE_STRIDE + 4 * (lane & 31));
             *reinterpret_cast<floatx4*>(o_rows + (size_t)r * D_V + 128 * ps + 4 * (lane & 31)) = v;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// 128 heads per workgroup, 8 wavefronts (two per SIMD).
+//
+// The per-head-group state of the kernel above (Q: 144 registers, O^T: 256) fills a SIMD's
+// whole register file with one wavefront, so nothing can overlap: MFMA, softmax arithmetic, LDS
+// reads and the issue of the gather loads simply add up, and four wavefronts do not issue
+// loads fast enough to keep HBM busy. Here each head group is a PAIR of wavefronts that splits
+// that state: wavefront (hg, dh) keeps the d-half `dh` of Q (72 registers) and the dv-half `dh`
+// of O^T (128 registers, ordinary VGPRs, so the running-max rescale is one multiply per
+// register). Per 32-row tile it computes the partial scores of its d-half (18 MFMAs), swaps
+// partials with its partner through LDS (4 KB each way), does the softmax on the full scores
+// (both partners get bit-identical results, the sum is taken in a fixed order), and multiplies
+// P with its half of V^T (16 MFMAs). No MFMA is duplicated, twice as many wavefronts issue
+// loads, and one wavefront's VALU/LDS phases overlap its SIMD neighbour's MFMAs.
+// ---------------------------------------------------------------------------------------------
+constexpr int HALF_K_STEPS = K_STEPS / 2;   // 18
+constexpr int HALF_DV_TILES = DV_TILES / 2;  // 8
+
+__device__ __forceinline__ void issue_tile_slice8(uint4* tile, const char* kv_b, const int* s_idx_tile,
+                                                  bool has_padding, int wave, int lane) {
+    // 36 load instructions per tile: wavefronts 0-3 issue 5 each, 4-7 issue 4 each
+    const int first = wave < 4 ? 5 * wave : 20 + 4 * (wave - 4);
+    const int count = wave < 4 ? 5 : 4;
+#pragma unroll
+    for (int i = 0; i < 5; ++i) {
+        if (i < count) {
+            int l = lane;
+            asm volatile("" : "+v"(l));
+            const int inst = first + i;
+            const int slot = inst * 64 + l;
+            const int row = slot / ROW_CHUNKS;
+            const int pos = slot - row * ROW_CHUNKS;
+            const int chunk = (pos & ~7) | ((pos ^ row) & 7);
+            const int key = s_idx_tile[row];
+            const char* src = kv_b + (size_t)(key < 0 ? 0 : key) * ROW_BYTES + chunk * 16;
+            const uint32_t lds_base = (uint32_t)(size_t)((lds_void_ptr)(tile + inst * 64));
+            if (!has_padding || key >= 0) {
+                asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off"
+                             :
+                             : "v"(src), "s"(lds_base)
+                             : "memory", "m0");
+            } else {
+                tile[slot] = make_uint4(0u, 0u, 0u, 0u);
+            }
+        }
+    }
+}
+
+// grid: x = split, y = request, z = group of 128 heads; 512 lanes
+__global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
+    const __bf16* __restrict__ q, const __bf16* __restrict__ kv, const int* __restrict__ idx,
+    float* __restrict__ o_part, float* __restrict__ lse_part, int n_heads, int n_kv_rows, int topk,
+    int rows_per_split, float scale_log2) {
+    typedef const __attribute__((address_space(3))) uintx4* lds_x4;
+    typedef shortx4 __attribute__((address_space(3)))* lds_s4;
+    __shared__ uint4 tiles[3 * TILE_CHUNKS];  // ring of three resident tiles
+    __shared__ floatx4 s_xchg[8][4 * 64];     // partial scores of every wavefront, 4 KB each
+    __shared__ int s_idx[MAX_SPLIT_ROWS];
+    __shared__ int s_first_masked_tile;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int hg = wave & 3;   // 32-head group
+    const int dh = wave >> 2;  // which half of d (QK^T) and of dv (PV) this wavefront owns
+    const int split = blockIdx.x;
+    const int n_splits = gridDim.x;
+    const int b = blockIdx.y;
+    const int head0 = blockIdx.z * 128 + hg * 32;
+    const int half = lane >> 5;
+
+    const int row_begin = split * rows_per_split;
+    int row_end = row_begin + rows_per_split;
+    if (row_end > topk) row_end = topk;
+    const int n_rows = row_end > row_begin ? row_end - row_begin : 0;
+    const int n_tiles = (n_rows + TILE_ROWS - 1) / TILE_ROWS;
+
+    // Q^T operand of this wavefront's share of d: local step l is k-step 4*(l/2) + 2*dh + l%2,
+    // i.e. the two wavefronts of a pair alternate 32-element slices of d
+    bf16x8 qreg[HALF_K_STEPS];
+    {
+        const __bf16* qrow = q + ((size_t)b * n_heads + head0 + (lane & 31)) * D_QK + 8 * half + 32 * dh;
+#pragma unroll
+        for (int l = 0; l < HALF_K_STEPS; ++l) {
+            qreg[l] = *reinterpret_cast<const bf16x8*>(qrow + 64 * (l >> 1) + 16 * (l & 1));
+        }
+    }
+
+    if (tid == 0) s_first_masked_tile = n_tiles;
+    __syncthreads();
+    for (int i = tid; i < n_tiles * TILE_ROWS; i += 512) {
+        int key = -1;
+        if (i < n_rows) {
+            key = idx[(size_t)b * topk + row_begin + i];
+            if (key >= n_kv_rows) key = -1;
+        }
+        if (key < 0) {
+            key = -1;
+            atomicMin(&s_first_masked_tile, i / TILE_ROWS);
+        }
+        s_idx[i] = key;
+    }
+    __syncthreads();
+    const int first_masked_tile = s_first_masked_tile;
+    const char* kv_b = reinterpret_cast<const char*>(kv) + (size_t)b * n_kv_rows * ROW_BYTES;
+
+    // Q has arrived before the first gather load is issued, so that no later wait for Q can
+    // drain the gather queue
+#pragma unroll
+    for (int ks = 0; ks < HALF_K_STEPS; ++ks) asm volatile("" : "+v"(qreg[ks]));
+    if (n_tiles > 0) issue_tile_slice8(tiles, kv_b, s_idx, 0 >= first_masked_tile, wave, lane);
+    if (n_tiles > 1) {
+        issue_tile_slice8(tiles + TILE_CHUNKS, kv_b, s_idx + TILE_ROWS, 1 >= first_masked_tile, wave, lane);
+    }
+
+
+    floatx16 acc[HALF_DV_TILES];
+#pragma unroll
+    for (int t = 0; t < HALF_DV_TILES; ++t) acc[t] = floatx16{0};
+    SoftmaxState st{-INFINITY, 0.f};
+    const LaneOffsets off = make_lane_offsets(lane);
+    // K operand of local step l: qk_l[l & 1] + (l >> 1) * 128
+    // V^T operand of local dv tile tl: pv_l[tl & 1] + (16*ks + 8*rr) * ROW_BYTES + (tl >> 1) * 128
+    const uint32_t qk_l[2] = {dh ? off.qk[2] : off.qk[0], dh ? off.qk[3] : off.qk[1]};
+    const uint32_t pv_l[2] = {off.pv[0] + 512u * dh, off.pv[1] + 512u * dh};
+    floatx4* my_xchg = &s_xchg[wave][0];
+    const floatx4* partner_xchg = &s_xchg[wave ^ 4][0];
+
+    // ring slots of tile t and of tile t+2 (wave-uniform, so the loop body exists once and the
+    // LDS addresses are a per-tile scalar added to the lane offsets)
+    int cur_slot = 0, fill_slot = 2;
+    for (int t = 0; t < n_tiles; ++t) {
+        const uint4* cur = tiles + cur_slot * TILE_CHUNKS;
+        uint4* nxt2 = tiles + fill_slot * TILE_CHUNKS;
+        cur_slot = cur_slot == 2 ? 0 : cur_slot + 1;
+        fill_slot = fill_slot == 2 ? 0 : fill_slot + 1;
+        // tile t resident for everybody, tile t-1 no longer read by anybody
+        const bool plain_wait = t + 1 < n_tiles && t + 1 < first_masked_tile;
+        if (plain_wait) {
+            if (wave < 4) wait_vmcnt<5>(); else wait_vmcnt<4>();
+        } else {
+            wait_all_memory();
+        }
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (t + 2 < n_tiles) {
+            issue_tile_slice8(nxt2, kv_b, s_idx + (t + 2) * TILE_ROWS, t + 2 >= first_masked_tile, wave, lane);
+        }
+        const lds_bytes base = (lds_bytes)cur;
+        const int* s_idx_tile = s_idx + t * TILE_ROWS;
+
+        // partial S^T over this wavefront's d-half
+        floatx16 s = {0};
+        {
+            uintx4 kbuf[2][2];
+            auto k_read = [&](int g) {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    kbuf[g & 1][j] = *(lds_x4)(base + qk_l[j] + g * 128);
+                }
+            };
+            k_read(0);
+#pragma unroll
+            for (int g = 0; g < HALF_K_STEPS / 2; ++g) {
+                if (g + 1 < HALF_K_STEPS / 2) k_read(g + 1);
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kbuf[g & 1][0]),
+                                                            qreg[2 * g], s, 0, 0, 0);
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kbuf[g & 1][1]),
+                                                            qreg[2 * g + 1], s, 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        // swap partials with the partner (same lane layout on both sides)
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+            my_xchg[qd * 64 + lane] = floatx4{s[4 * qd], s[4 * qd + 1], s[4 * qd + 2], s[4 * qd + 3]};
+        }
+        __builtin_amdgcn_s_waitcnt((63 & 15) | ((63 >> 4) << 14) | (7 << 4) | (0 << 8));  // lgkmcnt(0)
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+            const floatx4 o = partner_xchg[qd * 64 + lane];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                // fixed order (d-half 0 first) so that both partners compute identical sums
+                s[4 * qd + r] = dh == 0 ? s[4 * qd + r] + o[r] : o[r] + s[4 * qd + r];
+            }
+        }
+
+        // softmax on the tile's scores; register i of `s` is row 8*(i/4) + 4*half + i%4
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[i] *= scale_log2;
+        if (t >= first_masked_tile) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int row = 8 * (i / 4) + 4 * half + (i % 4);
+                if (s_idx_tile[row] < 0) s[i] = -INFINITY;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, s[i]);
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+        const bool move = tmax > st.m + FRAME_SLACK || st.m == -INFINITY;
+        const float m_new = move ? tmax : st.m;
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = move ? __builtin_amdgcn_exp2f(st.m - m_use) : 1.f;
+        const bool rescale = move && st.l != 0.f;
+        st.m = m_new;
+        float psum = 0.f;
+        bf16x8 p[2];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const __bf16 e = (__bf16)__builtin_amdgcn_exp2f(s[i] - m_use);
+            p[i / 8][i % 8] = e;
+            psum += (float)e;
+        }
+        st.l = st.l * alpha + psum;
+        if (__builtin_amdgcn_ballot_w64(rescale) != 0) {
+#pragma unroll
+            for (int tt = 0; tt < HALF_DV_TILES; ++tt) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) acc[tt][i] *= alpha;
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+
+        // O^T[dv half] += V^T P^T
+        shortx4 vbuf[2][2][2];
+        auto pv_read = [&](int stepi, shortx4 (&dst)[2][2]) {
+            // two MFMAs per group: (ks, dv tile) = stepi*2, stepi*2+1 in (ks major) order
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int idx2 = stepi * 2 + j;
+                const int ks = idx2 / HALF_DV_TILES;
+                const int tl = idx2 % HALF_DV_TILES;
+#pragma unroll
+                for (int rr = 0; rr < 2; ++rr) {
+                    dst[j][rr] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (lds_s4)(base + pv_l[tl & 1] + (16 * ks + 8 * rr) * ROW_BYTES + (tl >> 1) * 128));
+                }
+            }
+        };
+        pv_read(0, vbuf[0]);
+#pragma unroll
+        for (int g = 0; g < HALF_DV_TILES; ++g) {  // 8 groups of 2 MFMAs
+            if (g + 1 < HALF_DV_TILES) pv_read(g + 1, vbuf[(g + 1) & 1]);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int idx2 = g * 2 + j;
+                const int ks = idx2 / HALF_DV_TILES;
+                const int tl = idx2 % HALF_DV_TILES;
+                const bf16x4 lo = __builtin_bit_cast(bf16x4, vbuf[g & 1][j][0]);
+                const bf16x4 hi = __builtin_bit_cast(bf16x4, vbuf[g & 1][j][1]);
+                const bf16x8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                acc[tl] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, p[ks], acc[tl], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    // epilogue: normalise; O^T half -> LDS (64 dv at a time, region private to the wavefront)
+    // -> 256-byte row segments of the partial output
+    const float l_total = st.l + __shfl_xor(st.l, 32);
+    const float inv_l = l_total > 0.f ? 1.f / l_total : 0.f;
+    const size_t part0 = ((size_t)b * n_splits + split) * n_heads + head0;
+    if (dh == 0 && half == 0) {
+        lse_part[part0 + lane] = l_total > 0.f ? st.m + __builtin_amdgcn_logf(l_total) : -INFINITY;
+    }
+    __syncthreads();
+    constexpr int STAGE_STRIDE = 64 + 4;
+    float* stage = reinterpret_cast<float*>(tiles + (wave >> 2) * TILE_CHUNKS) + (wave & 3) * (32 * STAGE_STRIDE);
+    float* o_rows = o_part + part0 * D_V + 256 * dh;
+#pragma unroll
+    for (int ps = 0; ps < 4; ++ps) {
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+            const floatx16 a = acc[2 * ps + tt];
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd) {
+                floatx4 v = {a[4 * qd] * inv_l, a[4 * qd + 1] * inv_l, a[4 * qd + 2] * inv_l,
+                             a[4 * qd + 3] * inv_l};
+                *reinterpret_cast<floatx4*>(stage + (lane & 31) * STAGE_STRIDE + 32 * tt + 8 * qd +
+                                            4 * half) = v;
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            const int r = 4 * it + (lane >> 4);
+            const floatx4 v = *reinterpret_cast<const floatx4*>(stage + r * STAGE_STRIDE + 4 * (lane & 15));
+            *reinterpret_cast<floatx4*>(o_rows + (size_t)r * D_V + 64 * ps + 4 * (lane & 15)) = v;
         }
     }
 }
@@ -529,10 +831,14 @@ extern "C" void sparse_mla_decode_launcher(void* out, const void* q, const void*
         caa::set_status(CAA_BAD_ARGUMENT);
         return;
     }
-    if (workspace_bytes < sparse_mla_decode_workspace_bytes(batch, n_heads, topk, config)) {
+    if (workspace_bytes < sparse_mla_decode_workspace_bytes(batch, n_heads, topk, config % 1000)) {
         caa::set_status(CAA_WORKSPACE_TOO_SMALL);
         return;
     }
+    // config >= 1000: the one-wavefront-per-SIMD kernel for 128 heads (config - 1000 is then the
+    // split count)
+    const bool four_wave_kernel = config >= 1000;
+    if (four_wave_kernel) config -= 1000;
     const int head_groups = n_heads <= 128 ? 1 : n_heads / 128;
     const int splits = pick_splits(batch, head_groups, topk, config);
     const int tiles = (topk + TILE_ROWS - 1) / TILE_ROWS;
@@ -551,10 +857,13 @@ extern "C" void sparse_mla_decode_launcher(void* out, const void* q, const void*
         sparse_mla_split_kernel<2><<<grid, 128, 0, stream>>>(qb, kvb, idx, o_part, lse_part, n_heads,
                                                              n_kv_rows, topk, rows_per_split,
                                                              scale_log2);
-    } else {
+    } else if (four_wave_kernel) {
         sparse_mla_split_kernel<4><<<grid, 256, 0, stream>>>(qb, kvb, idx, o_part, lse_part, n_heads,
                                                              n_kv_rows, topk, rows_per_split,
                                                              scale_log2);
+    } else {
+        sparse_mla_split8_kernel<<<grid, 512, 0, stream>>>(qb, kvb, idx, o_part, lse_part, n_heads,
+                                                           n_kv_rows, topk, rows_per_split, scale_log2);
     }
     if (out_dtype == 0) {
         sparse_mla_merge_kernel<__bf16><<<dim3(n_heads, batch), 128, 0, stream>>>(
