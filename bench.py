@@ -34,10 +34,10 @@ FP8_PEAK_TFLOPS = 5033.0
 METRIC = "GB/s & % HBM peak (GDN/MoE/MLA decode); fp8 TFLOP/s % MFMA peak (MoE prefill)"
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled
-# by the same counters read on a plain 512 MiB copy kernel (FETCH_SIZE x 1.99982, WRITE_SIZE x 1,
-# both in KiB); the counter summary is profiles/gdn_mla_moe_decode_hbm_traffic_pmc.md.
+# by the same counters read on a plain 512 MiB copy kernel (FETCH_SIZE x 1.99984, WRITE_SIZE x 1,
+# both in KiB); the counter summary is profiles/all_workloads_hbm_traffic_pmc.md.
 # None = not measured.
-MEASURED_TRAFFIC = {'gdn': 1086006640, 'moe_decode': 6703804038, 'mla': 259340846, 'moe_prefill': None}
+MEASURED_TRAFFIC = {'gdn': 1085986734, 'moe_decode': 6664742582, 'mla': 277476469, 'moe_prefill': 11202932427}
 
 
 def timed_launches(torch, launch, steps, warmup):
@@ -119,7 +119,7 @@ def bench_mla(torch, capi, dev, steps, warmup, cpu_baseline):
     res = dict(
         workload="configs[3]: sparse-MLA decode B=64, 128 heads, 576-dim latent rows, top-k 2048 of 32768, "
                  "bf16, seed 20253 (split kernel + merge per step)",
-        value=work / sec / 1e9, unit="GB/s", ms_per_step=sec * 1e3, dtype="bf16", kernel="sparse_mla_split_kernel",
+        value=work / sec / 1e9, unit="GB/s", ms_per_step=sec * 1e3, dtype="bf16", kernel="sparse_mla_split8_kernel",
         roofline=dict(bound="hbm", achieved=work / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
                       frac=work / sec / 1e9 / HBM_PEAK_GBS, traffic=MEASURED_TRAFFIC['mla']),
         algorithmic_bytes=work, tflops=flops / sec / 1e12)
@@ -187,7 +187,7 @@ def bench_moe(torch, capi, dev, steps, warmup, cpu_baseline, prefill):
             workload="configs[4]: FP8 MoE prefill T=8192, hidden 7168, 256 experts x inter 2048, top-8, +2 logit "
                      "bias on 16 experts, e4m3 with 128x128 block scales, seed 20254 (whole layer per step)",
             value=flops / sec / 1e12, unit="TFLOP/s", ms_per_step=sec * 1e3, dtype="f8e4m3",
-            kernel="moe_stream_gemm_kernel",
+            kernel="moe_tiled_gemm_kernel",
             roofline=dict(bound="mfma", achieved=flops / sec / 1e12, peak=FP8_PEAK_TFLOPS, unit="TFLOP/s",
                           frac=flops / sec / 1e12 / FP8_PEAK_TFLOPS, traffic=MEASURED_TRAFFIC['moe_prefill']),
             algorithmic_flops=flops, active_experts=n_active)
@@ -196,7 +196,7 @@ def bench_moe(torch, capi, dev, steps, warmup, cpu_baseline, prefill):
             workload="configs[2]: FP8 MoE decode T=64, hidden 7168, 256 experts x inter 2048, top-8, e4m3 with "
                      "128x128 block scales, seed 20252 (whole layer per step)",
             value=wbytes / sec / 1e9, unit="GB/s", ms_per_step=sec * 1e3, dtype="f8e4m3",
-            kernel="moe_stream_gemm_kernel",
+            kernel="moe_stream_gemm_lds_kernel",
             roofline=dict(bound="hbm", achieved=wbytes / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
                           frac=wbytes / sec / 1e9 / HBM_PEAK_GBS, traffic=MEASURED_TRAFFIC['moe_decode']),
             algorithmic_bytes=wbytes, active_experts=n_active, tflops=flops / sec / 1e12)
