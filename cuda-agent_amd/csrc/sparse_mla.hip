@@ -447,46 +447,83 @@ __global__ __launch_bounds__(64 * NW) void sparse_mla_split_kernel(
 //
 // The per-head-group state of the kernel above (Q: 144 registers, O^T: 256) fills a SIMD's
 // whole register file with one wavefront, so nothing can overlap: MFMA, softmax arithmetic, LDS
-// reads and the issue of the gather loads simply add up, and four wavefronts do not issue
-// loads fast enough to keep HBM busy. Here each head group is a PAIR of wavefronts that splits
-// that state: wavefront (hg, dh) keeps the d-half `dh` of Q (72 registers) and the dv-half `dh`
-// of O^T (128 registers, ordinary VGPRs, so the running-max rescale is one multiply per
-// register). Per 32-row tile it computes the partial scores of its d-half (18 MFMAs), swaps
-// partials with its partner through LDS (4 KB each way), does the softmax on the full scores
-// (both partners get bit-identical results, the sum is taken in a fixed order), and multiplies
-// P with its half of V^T (16 MFMAs). No MFMA is duplicated, twice as many wavefronts issue
-// loads, and one wavefront's VALU/LDS phases overlap its SIMD neighbour's MFMAs.
+// reads and the issue of the gather loads simply add up. Here each head group is a PAIR of
+// wavefronts (w, w^1, on different SIMDs) that splits that state: each keeps alternating
+// 32-element slices of d of Q (72 registers) and one half of dv of O^T (128 registers, ordinary
+// VGPRs, so the running-max rescale is one multiply per register). Per 32-row tile a wavefront
+// computes the partial scores of its d slices (18 MFMAs) into an exchange buffer in LDS; after a
+// workgroup barrier both partners add the two partials in the same order, do the softmax on the
+// full scores (bit-identical in both) and multiply P with their half of V^T (16 MFMAs). No MFMA
+// is duplicated.
+// Wavefronts 0-3 (lead) and 4-7 (lag; w and w+4 share a SIMD) run half a tile apart, so that on
+// every SIMD one wavefront is in its QK^T half-step while the other is in its softmax/PV
+// half-step. The lag group also gathers: each of its wavefronts loads 8 whole rows of a tile.
+// Measured per wavefront and tile (core clock cycles, 16-tile splits): gather issue 2 000 (the
+// memory pipeline accepts one 1 KB load of a wavefront per 150-300 cycles, whatever the
+// addresses), QK^T 950-1 200, softmax + rescale 1 750-1 950, PV 650-900, barriers 500-2 800;
+// the prologue (indices, Q, first tiles) is 10 us and the epilogue (262 KB of partials) 5 us.
 // ---------------------------------------------------------------------------------------------
+// Phase timing build (-DMLA_PHASE_TIMING): every wavefront of workgroup (0,0,0) adds up the core
+// clock cycles it spends in each phase of the loop and leaves them in g_phase_cycles.
+#ifdef MLA_PHASE_TIMING
+__device__ unsigned long long g_phase_cycles[8][12];
+#define PHASE_TIMING_BEGIN() unsigned long long phase_t0 = __builtin_readcyclecounter(), phase_acc[12] = {}
+#define PHASE_MARK(n)                                                    \
+    {                                                                    \
+        const unsigned long long phase_now = __builtin_readcyclecounter(); \
+        phase_acc[n] += phase_now - phase_t0;                            \
+        phase_t0 = phase_now;                                            \
+    }
+#define PHASE_TIMING_END(wave, lane)                                                     \
+    if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && (lane) == 0) {          \
+        for (int i = 0; i < 11; ++i) g_phase_cycles[wave][i] = phase_acc[i];             \
+        g_phase_cycles[wave][11] = __builtin_amdgcn_s_getreg((31 << 11) | 4); /* HW_ID */ \
+    }
+#else
+#define PHASE_TIMING_BEGIN()
+#define PHASE_MARK(n)
+#define PHASE_TIMING_END(wave, lane)
+#endif
+
 constexpr int HALF_K_STEPS = K_STEPS / 2;   // 18
 constexpr int HALF_DV_TILES = DV_TILES / 2;  // 8
 
-__device__ __forceinline__ void issue_tile_slice8(uint4* tile, const char* kv_b, const int* s_idx_tile,
-                                                  bool has_padding, int wave, int lane) {
-    // 36 load instructions per tile: wavefronts 0-3 issue 5 each, 4-7 issue 4 each
-    const int first = wave < 4 ? 5 * wave : 20 + 4 * (wave - 4);
-    const int count = wave < 4 ? 5 : 4;
+// Gather of one tile by the four wavefronts of the lag group: wavefront `quarter` loads rows
+// 8*quarter .. 8*quarter+7, which are 576 16-byte chunks = exactly 9 load instructions. `tab`
+// holds, for chunk c = 64*i + lane of that span, (4 * (c / 72)) << 16 | byte offset of the
+// swizzled source chunk within the row; it is the same for every tile and every wavefront.
+// The loads address the request's cache block as 64-bit scalar base + 32-bit lane offset, so a
+// prepared tile costs 9 registers; gather_prepare() reads table and indices for all nine loads
+// at once, so that the nine address chains overlap.
+constexpr int GATHER_INSTR = 9;
+constexpr int GATHER_TAB = GATHER_INSTR * 64;
+constexpr uint32_t GATHER_MASKED = 0xffffffffu;  // offset sentinel of a padding row
+
+__device__ __forceinline__ void gather_prepare(uint32_t (&off)[GATHER_INSTR], const int* s_idx_tile,
+                                               const uint32_t* tab, bool has_padding, int quarter, int lane) {
+    const char* keys = reinterpret_cast<const char*>(s_idx_tile + 8 * quarter);
+    uint32_t e[GATHER_INSTR];
 #pragma unroll
-    for (int i = 0; i < 5; ++i) {
-        if (i < count) {
-            int l = lane;
-            asm volatile("" : "+v"(l));
-            const int inst = first + i;
-            const int slot = inst * 64 + l;
-            const int row = slot / ROW_CHUNKS;
-            const int pos = slot - row * ROW_CHUNKS;
-            const int chunk = (pos & ~7) | ((pos ^ row) & 7);
-            const int key = s_idx_tile[row];
-            const char* src = kv_b + (size_t)(key < 0 ? 0 : key) * ROW_BYTES + chunk * 16;
-            const uint32_t lds_base = (uint32_t)(size_t)((lds_void_ptr)(tile + inst * 64));
-            if (!has_padding || key >= 0) {
-                asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off"
-                             :
-                             : "v"(src), "s"(lds_base)
-                             : "memory", "m0");
-            } else {
-                tile[slot] = make_uint4(0u, 0u, 0u, 0u);
-            }
-        }
+    for (int i = 0; i < GATHER_INSTR; ++i) e[i] = tab[64 * i + lane];
+#pragma unroll
+    for (int i = 0; i < GATHER_INSTR; ++i) {
+        const int key = *reinterpret_cast<const int*>(keys + (e[i] >> 16));
+        off[i] = (uint32_t)key * (uint32_t)ROW_BYTES + (e[i] & 0xffffu);
+        if (has_padding && key < 0) off[i] = GATHER_MASKED;
+    }
+}
+
+__device__ __forceinline__ void gather_issue(uint4* tile, const char* kv_b, uint32_t off, int i,
+                                             bool has_padding, int quarter, int lane) {
+    uint4* dst = tile + quarter * GATHER_TAB + i * 64;
+    if (!has_padding || off != GATHER_MASKED) {
+        const uint32_t lds_base = (uint32_t)(size_t)((lds_void_ptr)dst);
+        asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :
+                     : "v"(off), "s"(kv_b), "s"(lds_base)
+                     : "memory", "m0");
+    } else {
+        dst[lane] = make_uint4(0u, 0u, 0u, 0u);
     }
 }
 
@@ -500,13 +537,18 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
     __shared__ uint4 tiles[3 * TILE_CHUNKS];  // ring of three resident tiles
     __shared__ floatx4 s_xchg[8][4 * 64];     // partial scores of every wavefront, 4 KB each
     __shared__ int s_idx[MAX_SPLIT_ROWS];
+    __shared__ uint32_t s_gather_tab[GATHER_TAB];
     __shared__ int s_first_masked_tile;
 
+    PHASE_TIMING_BEGIN();
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int hg = wave & 3;   // 32-head group
-    const int dh = wave >> 2;  // which half of d (QK^T) and of dv (PV) this wavefront owns
+    // wavefronts w and w^1 are a pair (they sit on different SIMDs); wavefronts w and w+4 share
+    // a SIMD and belong to the lead (0-3) and the lag (4-7) group
+    const int dh = wave & 1;   // which slices of d (QK^T) and which half of dv (PV) this wavefront owns
+    const int hg = wave >> 1;  // 32-head group
+    const int group = wave >> 2;
     const int split = blockIdx.x;
     const int n_splits = gridDim.x;
     const int b = blockIdx.y;
@@ -519,8 +561,55 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
     const int n_rows = row_end > row_begin ? row_end - row_begin : 0;
     const int n_tiles = (n_rows + TILE_ROWS - 1) / TILE_ROWS;
 
+    // indices of the split first: everything else in the prologue queues up behind them
+    int raw_key[MAX_SPLIT_ROWS / 512];
+#pragma unroll
+    for (int j = 0; j < MAX_SPLIT_ROWS / 512; ++j) {
+        const int i = tid + 512 * j;
+        raw_key[j] = i < n_rows ? idx[(size_t)b * topk + row_begin + i] : -1;
+    }
+    if (tid == 0) s_first_masked_tile = n_tiles;
+    for (int c = tid; c < GATHER_TAB; c += 512) {
+        const int row = c / ROW_CHUNKS;  // 0..7; the tile row is 8*quarter + row, same low 3 bits
+        const int pos = c - row * ROW_CHUNKS;
+        const int chunk = (pos & ~7) | ((pos ^ row) & 7);
+        s_gather_tab[c] = ((uint32_t)(4 * row) << 16) | (uint32_t)(chunk * 16);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < MAX_SPLIT_ROWS / 512; ++j) {
+        const int i = tid + 512 * j;
+        if (i < n_tiles * TILE_ROWS) {
+            int key = raw_key[j];
+            if (key < 0 || key >= n_kv_rows) {
+                key = -1;
+                atomicMin(&s_first_masked_tile, i / TILE_ROWS);
+            }
+            s_idx[i] = key;
+        }
+    }
+    __syncthreads();
+    const int first_masked_tile = s_first_masked_tile;
+    const char* kv_b = reinterpret_cast<const char*>(kv) + (size_t)b * n_kv_rows * ROW_BYTES;
+    PHASE_MARK(7);  // index staging
+
+    // The first two tiles are on their way before Q is fetched: tile 0 by the lead group, tile 1
+    // by the lag group (a cold load instruction takes several hundred cycles to issue, so the
+    // two groups share the work; from tile 2 on the lag group gathers alone).
+    if (group < n_tiles) {
+        uint32_t off[GATHER_INSTR];
+        const bool pad = group >= first_masked_tile;
+        gather_prepare(off, s_idx + group * TILE_ROWS, s_gather_tab, pad, wave & 3, lane);
+#pragma unroll
+        for (int i = 0; i < GATHER_INSTR; ++i) {
+            gather_issue(tiles + group * TILE_CHUNKS, kv_b, off[i], i, pad, wave & 3, lane);
+        }
+    }
+    PHASE_MARK(9);  // first gather issue
+
     // Q^T operand of this wavefront's share of d: local step l is k-step 4*(l/2) + 2*dh + l%2,
-    // i.e. the two wavefronts of a pair alternate 32-element slices of d
+    // i.e. the two wavefronts of a pair alternate 32-element slices of d. The wait for Q also
+    // waits for the two tiles issued above (loads return in order), which the loop needs anyway.
     bf16x8 qreg[HALF_K_STEPS];
     {
         const __bf16* qrow = q + ((size_t)b * n_heads + head0 + (lane & 31)) * D_QK + 8 * half + 32 * dh;
@@ -529,34 +618,9 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
             qreg[l] = *reinterpret_cast<const bf16x8*>(qrow + 64 * (l >> 1) + 16 * (l & 1));
         }
     }
-
-    if (tid == 0) s_first_masked_tile = n_tiles;
-    __syncthreads();
-    for (int i = tid; i < n_tiles * TILE_ROWS; i += 512) {
-        int key = -1;
-        if (i < n_rows) {
-            key = idx[(size_t)b * topk + row_begin + i];
-            if (key >= n_kv_rows) key = -1;
-        }
-        if (key < 0) {
-            key = -1;
-            atomicMin(&s_first_masked_tile, i / TILE_ROWS);
-        }
-        s_idx[i] = key;
-    }
-    __syncthreads();
-    const int first_masked_tile = s_first_masked_tile;
-    const char* kv_b = reinterpret_cast<const char*>(kv) + (size_t)b * n_kv_rows * ROW_BYTES;
-
-    // Q has arrived before the first gather load is issued, so that no later wait for Q can
-    // drain the gather queue
 #pragma unroll
     for (int ks = 0; ks < HALF_K_STEPS; ++ks) asm volatile("" : "+v"(qreg[ks]));
-    if (n_tiles > 0) issue_tile_slice8(tiles, kv_b, s_idx, 0 >= first_masked_tile, wave, lane);
-    if (n_tiles > 1) {
-        issue_tile_slice8(tiles + TILE_CHUNKS, kv_b, s_idx + TILE_ROWS, 1 >= first_masked_tile, wave, lane);
-    }
-
+    PHASE_MARK(8);  // wait for Q
 
     floatx16 acc[HALF_DV_TILES];
 #pragma unroll
@@ -568,74 +632,93 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
     const uint32_t qk_l[2] = {dh ? off.qk[2] : off.qk[0], dh ? off.qk[3] : off.qk[1]};
     const uint32_t pv_l[2] = {off.pv[0] + 512u * dh, off.pv[1] + 512u * dh};
     floatx4* my_xchg = &s_xchg[wave][0];
-    const floatx4* partner_xchg = &s_xchg[wave ^ 4][0];
+    const floatx4* pair_xchg = &s_xchg[wave & ~1][0];  // d-slices 0 partial, then d-slices 1 partial
 
-    // ring slots of tile t and of tile t+2 (wave-uniform, so the loop body exists once and the
-    // LDS addresses are a per-tile scalar added to the lane offsets)
-    int cur_slot = 0, fill_slot = 2;
-    for (int t = 0; t < n_tiles; ++t) {
-        const uint4* cur = tiles + cur_slot * TILE_CHUNKS;
-        uint4* nxt2 = tiles + fill_slot * TILE_CHUNKS;
-        cur_slot = cur_slot == 2 ? 0 : cur_slot + 1;
-        fill_slot = fill_slot == 2 ? 0 : fill_slot + 1;
-        // tile t resident for everybody, tile t-1 no longer read by anybody
-        const bool plain_wait = t + 1 < n_tiles && t + 1 < first_masked_tile;
-        if (plain_wait) {
-            if (wave < 4) wait_vmcnt<5>(); else wait_vmcnt<4>();
-        } else {
-            wait_all_memory();
-        }
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-        if (t + 2 < n_tiles) {
-            issue_tile_slice8(nxt2, kv_b, s_idx + (t + 2) * TILE_ROWS, t + 2 >= first_masked_tile, wave, lane);
-        }
-        const lds_bytes base = (lds_bytes)cur;
-        const int* s_idx_tile = s_idx + t * TILE_ROWS;
-
-        // partial S^T over this wavefront's d-half
-        floatx16 s = {0};
-        {
-            uintx4 kbuf[2][2];
-            auto k_read = [&](int g) {
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    kbuf[g & 1][j] = *(lds_x4)(base + qk_l[j] + g * 128);
-                }
-            };
-            k_read(0);
-#pragma unroll
-            for (int g = 0; g < HALF_K_STEPS / 2; ++g) {
-                if (g + 1 < HALF_K_STEPS / 2) k_read(g + 1);
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kbuf[g & 1][0]),
-                                                            qreg[2 * g], s, 0, 0, 0);
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kbuf[g & 1][1]),
-                                                            qreg[2 * g + 1], s, 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
+    // The loop runs in half-steps with one workgroup barrier each. A wavefront alternates between
+    // a QK^T half-step (partial scores of one tile into its exchange buffer) and a softmax + PV
+    // half-step (which starts by reading both partners' partials, so the exchange crosses exactly
+    // one barrier). The lag group runs one half-step behind the lead group: on every SIMD one
+    // wavefront is in its MFMA-bound phase while the other is in its VALU-bound phase.
+    //   half-step h, lead: h even -> QK^T(h/2), h odd -> softmax/PV((h-1)/2)
+    //                lag:  h odd  -> QK^T((h-1)/2), h even -> softmax/PV(h/2 - 1)
+    // Tile t is last read in half-step 2t+2, so its ring slot is refilled (tile t+3) after the
+    // barrier of half-step 2t+3.
+    for (int h = 0; h <= 2 * n_tiles; ++h) {
+        PHASE_MARK(6);
+        if ((h & 1) == 0 && h < 2 * n_tiles) {
+            // tile h/2 must be resident: everything but this wavefront's share of the next tile
+            const int t = h >> 1;
+            const bool plain_wait = t + 1 < n_tiles && t + 1 < first_masked_tile;
+            if (plain_wait) {
+                wait_vmcnt<GATHER_INSTR>();  // (the lead group has no loads in flight)
+            } else {
+                wait_all_memory();
             }
-        }
-        // swap partials with the partner (same lane layout on both sides)
-#pragma unroll
-        for (int qd = 0; qd < 4; ++qd) {
-            my_xchg[qd * 64 + lane] = floatx4{s[4 * qd], s[4 * qd + 1], s[4 * qd + 2], s[4 * qd + 3]};
         }
         __builtin_amdgcn_s_waitcnt((63 & 15) | ((63 >> 4) << 14) | (7 << 4) | (0 << 8));  // lgkmcnt(0)
+        PHASE_MARK(0);  // wait for this wavefront's own gather loads and LDS stores
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
+        PHASE_MARK(1);  // wait for the other wavefronts
+        // the lag group's QK^T half-steps (odd h) also gather tile (h-1)/2 + 2 into the slot
+        // that tile (h-1)/2 - 1 has left after the barrier above
+        const int t2 = (h >> 1) + 2;
+        const bool gather = (h & 1) && group == 1 && t2 < n_tiles;
+        const bool gather_pad = t2 >= first_masked_tile;
+        uint4* gather_tile = tiles + ((gather ? t2 : 0) % 3) * TILE_CHUNKS;
+        const int mine = h - group;  // this wavefront's own half-step counter
+        const int t = mine >> 1;
+        const bool active = mine >= 0 && t < n_tiles;
+        const lds_bytes base = (lds_bytes)(tiles + ((active ? t : 0) % 3) * TILE_CHUNKS);
+
+        if (active && (mine & 1) == 0) {
+            // partial S^T over this wavefront's slices of d
+            floatx16 s = {0};
+            // Gather of tile t2 first: the memory pipeline takes the nine loads of a wavefront
+            // at one per ~150 cycles whether or not MFMAs are issued in between (measured), so
+            // they go out back to back and the QK^T loop stays free of them.
+            if (gather) {
+                uint32_t goff[GATHER_INSTR];
+                gather_prepare(goff, s_idx + t2 * TILE_ROWS, s_gather_tab, gather_pad, wave & 3, lane);
+#pragma unroll
+                for (int i = 0; i < GATHER_INSTR; ++i) {
+                    gather_issue(gather_tile, kv_b, goff[i], i, gather_pad, wave & 3, lane);
+                }
+            }
+            PHASE_MARK(2);  // gather issue
+            uintx4 kbuf[3];  // K operands are read two MFMAs ahead
+            auto k_read = [&](int l) { kbuf[l % 3] = *(lds_x4)(base + qk_l[l & 1] + (l >> 1) * 128); };
+            k_read(0);
+            k_read(1);
+#pragma unroll
+            for (int l = 0; l < HALF_K_STEPS; ++l) {
+                if (l + 2 < HALF_K_STEPS) k_read(l + 2);
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kbuf[l % 3]), qreg[l], s,
+                                                            0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd) {
+                my_xchg[qd * 64 + lane] = floatx4{s[4 * qd], s[4 * qd + 1], s[4 * qd + 2], s[4 * qd + 3]};
+            }
+            PHASE_MARK(3);  // QK^T
+        }
+        if (!(active && (mine & 1) == 1)) continue;
+
+        // full scores = partial of d-slices 0 + partial of d-slices 1, in that order in both
+        // partners, so that they compute bit-identical probabilities
+        const int* s_idx_tile = s_idx + t * TILE_ROWS;
+        floatx16 s;
 #pragma unroll
         for (int qd = 0; qd < 4; ++qd) {
-            const floatx4 o = partner_xchg[qd * 64 + lane];
+            const floatx4 lo = pair_xchg[qd * 64 + lane];
+            const floatx4 hi = pair_xchg[4 * 64 + qd * 64 + lane];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                // fixed order (d-half 0 first) so that both partners compute identical sums
-                s[4 * qd + r] = dh == 0 ? s[4 * qd + r] + o[r] : o[r] + s[4 * qd + r];
-            }
+            for (int r = 0; r < 4; ++r) s[4 * qd + r] = (lo[r] + hi[r]) * scale_log2;
         }
 
         // softmax on the tile's scores; register i of `s` is row 8*(i/4) + 4*half + i%4
         float tmax = -INFINITY;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) s[i] *= scale_log2;
         if (t >= first_masked_tile) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
@@ -669,6 +752,7 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
             }
         }
         __builtin_amdgcn_sched_barrier(0);
+        PHASE_MARK(4);  // exchange read, softmax, rescale
 
         // O^T[dv half] += V^T P^T
         shortx4 vbuf[2][2][2];
@@ -702,6 +786,7 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
             }
             __builtin_amdgcn_sched_barrier(0);
         }
+        PHASE_MARK(5);  // PV
     }
 
     // epilogue: normalise; O^T half -> LDS (64 dv at a time, region private to the wavefront)
@@ -736,6 +821,8 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
             *reinterpret_cast<floatx4*>(o_rows + (size_t)r * D_V + 64 * ps + 4 * (lane & 15)) = v;
         }
     }
+    PHASE_MARK(10);  // epilogue
+    PHASE_TIMING_END(wave, lane);
 }
 
 // out[b, h, :] = sum_s w_s o_part[b, s, h, :],  w_s = exp2(lse_s - max) / sum; one workgroup of
@@ -837,8 +924,10 @@ extern "C" void sparse_mla_decode_launcher(void* out, const void* q, const void*
     }
     // config >= 1000: the one-wavefront-per-SIMD kernel for 128 heads (config - 1000 is then the
     // split count)
-    const bool four_wave_kernel = config >= 1000;
-    if (four_wave_kernel) config -= 1000;
+    // The 8-wavefront kernel addresses a request's cache block with 32-bit byte offsets.
+    const bool four_wave_kernel =
+        config >= 1000 || (unsigned long long)n_kv_rows * ROW_BYTES >= 0xffffffffull;
+    if (config >= 1000) config -= 1000;
     const int head_groups = n_heads <= 128 ? 1 : n_heads / 128;
     const int splits = pick_splits(batch, head_groups, topk, config);
     const int tiles = (topk + TILE_ROWS - 1) / TILE_ROWS;
