@@ -49,6 +49,11 @@ inline int tiled_grid(int row_tiles, int max_pair_tiles) {
     return ((supers + 7) / 8) * 8 * SUPER_ROWS * SUPER_PAIRS;
 }
 
+template <int N>
+struct IntConstant {
+    static constexpr int value = N;
+};
+
 __device__ __forceinline__ intx8 join(intx4 lo, intx4 hi) {
     return intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
 }
@@ -102,6 +107,27 @@ __global__ __launch_bounds__(256) void moe_gather_scales_kernel(const float* __r
     }
 }
 
+// Phase timing build (-DMOE_PHASE_TIMING): every wavefront of workgroup 0 adds up the core clock
+// cycles it spends in each phase of the K loop and leaves them in g_phase_cycles.
+#ifdef MOE_PHASE_TIMING
+__device__ unsigned long long g_phase_cycles[8][8];
+#define PHASE_TIMING_BEGIN() unsigned long long phase_t0 = __builtin_readcyclecounter(), phase_acc[8] = {}
+#define PHASE_MARK(n)                                                      \
+    {                                                                      \
+        const unsigned long long phase_now = __builtin_readcyclecounter(); \
+        phase_acc[n] += phase_now - phase_t0;                              \
+        phase_t0 = phase_now;                                              \
+    }
+#define PHASE_TIMING_END(wave, lane)                                        \
+    if (blockIdx.x == 0 && (lane) == 0) {                                   \
+        for (int i = 0; i < 8; ++i) g_phase_cycles[wave][i] = phase_acc[i]; \
+    }
+#else
+#define PHASE_TIMING_BEGIN()
+#define PHASE_MARK(n)
+#define PHASE_TIMING_END(wave, lane)
+#endif
+
 // grid: 1-D, see the mapping at the top of the kernel
 template <bool GATE_UP>
 __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
@@ -151,7 +177,7 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
     const uint32_t ld_chunk = (lane & 7) ^ ld_row;
     const uint32_t ld_off = ld_row * (uint32_t)K + 16 * ld_chunk;
     const uint8_t* a_src[4];
-    const uint8_t* b_src[4];
+    uint32_t b_off[4];  // byte offset of this lane's activation row and chunk (the buffers are < 4 GB)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int ar = (4 * wave + i) * 8;  // first of the 8 tile rows of this instruction
@@ -162,7 +188,7 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
         int p = (4 * wave + i) * 8 + (int)ld_row;
         p = begin + (p < cnt ? p : cnt - 1);  // rows past the tile's end repeat the last one
         const int arow = GATE_UP ? sorted_pairs[p] / top_k : p;
-        b_src[i] = a_q + (size_t)arow * K + 16 * ld_chunk;
+        b_off[i] = (uint32_t)arow * (uint32_t)K + 16 * ld_chunk;
     }
     const float* s_src = as_t + begin;  // + kb*scale_stride; 256 floats, the tail is padding
     const float* ws0;
@@ -176,16 +202,18 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
     }
 
     const uint32_t stage_base = (uint32_t)(size_t)((lds_void_ptr)s_stage);
-    auto issue_stage = [&](int kb) {
-        const uint32_t st = stage_base + (kb & 1) * STAGE_BYTES;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
+    // load i (0..7) of this wavefront's share of stage kb: 0..3 weights, 4..7 activations
+    auto issue_load = [&](int kb, int i, int slot_parity) {
+        const uint32_t st = stage_base + (slot_parity & 1) * STAGE_BYTES;
+        if (i < 4) {
             dma16(a_src[i] + (size_t)kb * GROUP, ld_off, st + (4 * wave + i) * 1024);
-            dma16_ptr(b_src[i] + (size_t)kb * GROUP, st + STAGE_A + (4 * wave + i) * 1024);
+        } else {
+            dma16(a_q + (size_t)kb * GROUP, b_off[i - 4], st + STAGE_A + (4 * wave + i - 4) * 1024);
         }
-        if (wave == 0) {
-            dma16(s_src + (size_t)kb * scale_stride, lane * 16, st + STAGE_A + STAGE_B);
-        }
+    };
+    auto issue_scales = [&](int kb, int slot_parity) {
+        const uint32_t st = stage_base + (slot_parity & 1) * STAGE_BYTES;
+        if (wave == 0) dma16(s_src + (size_t)kb * scale_stride, lane * 16, st + STAGE_A + STAGE_B);
     };
 
     // ---- read side -------------------------------------------------------------------------
@@ -204,45 +232,139 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
 #pragma unroll
         for (int b = 0; b < 4; ++b) acc[a][b] = floatx16{0};
 
-    issue_stage(0);
-    for (int kb = 0; kb < KB; ++kb) {
-        wait_all_loads();
+    // One K block for a wavefront with NB (compile time) active B tiles.
+    //  * Weights are in flight for two blocks, activations for one. A wavefront copies its A
+    //    operands of the block into registers at the top, so after a second barrier the weight
+    //    half of the stage is free again and the weights of block kb+2 are loaded into it, while
+    //    the activations and pair scales of block kb+1 go to the other stage. One stage in
+    //    flight (65 KB per CU) at 1.5-2 us of loaded HBM latency was 35 GB/s per CU and bound the
+    //    kernel; weights are the part that comes from HBM.
+    //  * The activation loads are issued before the weight loads, so "at most 4 loads
+    //    outstanding" at the top of a block means everything but the weights of block kb+1.
+    //  * The loads go out between MFMA pairs (a load holds the wavefront for 60-130 cycles until
+    //    the memory pipeline has taken it).
+    //  * The next B tile is read from LDS as soon as the last MFMA of the current one has been
+    //    issued; the partial of A tile 0 is promoted (acc += partial * scale) while the MFMAs of
+    //    A tile 1 run, and the partial of A tile 1 while the next step's first MFMAs run, so the
+    //    VALU work hides behind the matrix pipeline with two partial accumulators only.
+    // kb1, kb2: kb+1 and kb+2, or 0 past the end (harmless loads that keep the body branch-free;
+    // the epilogue waits for them before it reuses the stages).
+    auto block = [&](auto nb_tag, int kb, int kb1, int kb2) {
+        constexpr int NB = decltype(nb_tag)::value;
+        const lds_bytes st = stage_ptr + (kb & 1) * STAGE_BYTES;
+        intx8 A[2][2];  // [tile][k-step]
+        intx8 B[2];     // [k-step]
+        float bs = 0.f;
+        auto read_b = [&](int b) {
+            const lds_bytes bt = st + STAGE_A + (th * 128 + b * 32) * GROUP;
+            B[0] = join(*(lds_x4)(bt + rd), *(lds_x4)(bt + (rd ^ 16)));
+            B[1] = join(*(lds_x4)(bt + (rd ^ 64)), *(lds_x4)(bt + (rd ^ 64 ^ 16)));
+        };
+        auto read_bs = [&](int b) {
+            return *(const __attribute__((address_space(3))) float*)(st + STAGE_A + STAGE_B +
+                                                                     (th * 128 + b * 32 + r32) * 4);
+        };
+        if (NB > 0) {
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                A[0][s] = join(*(lds_x4)(st + a_row0 * GROUP + (rd ^ (64 * s))),
+                               *(lds_x4)(st + a_row0 * GROUP + (rd ^ (64 * s) ^ 16)));
+                A[1][s] = join(*(lds_x4)(st + a_row1 * GROUP + (rd ^ (64 * s))),
+                               *(lds_x4)(st + a_row1 * GROUP + (rd ^ (64 * s) ^ 16)));
+            }
+            read_b(0);
+            bs = read_bs(0);
+        }
+        issue_scales(kb1, kb + 1);
+#pragma unroll
+        for (int i = 4; i < 8; ++i) issue_load(kb1, i, kb + 1);
+        // every wavefront holds its A operands: the weight half of this stage may be refilled
+        __builtin_amdgcn_s_waitcnt((63 & 15) | ((63 >> 4) << 14) | (7 << 4) | (0 << 8));  // lgkmcnt(0)
+        asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        if (kb + 1 < KB) issue_stage(kb + 1);
-
-        const lds_bytes st = stage_ptr + (kb & 1) * STAGE_BYTES;
+        constexpr int PER_SLOT = NB >= 2 ? 1 : NB == 1 ? 2 : 4;  // weight loads per MFMA pair
+        auto loads = [&](int slot) {
+#pragma unroll
+            for (int j = 0; j < PER_SLOT; ++j) {
+                const int i = slot * PER_SLOT + j;
+                if (i < 4) issue_load(kb2, i, kb);
+            }
+        };
+        if (NB == 0) {
+            loads(0);
+            return;
+        }
         const float w0 = ws0[kb];
         const float w1 = ws1[kb];
-        intx8 A[2][2];  // [tile][k-step]
+        floatx16 p0, p1;
+        float s1_prev = 0.f;
 #pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            A[0][s] = join(*(lds_x4)(st + a_row0 * GROUP + (rd ^ (64 * s))),
-                           *(lds_x4)(st + a_row0 * GROUP + (rd ^ (64 * s) ^ 16)));
-            A[1][s] = join(*(lds_x4)(st + a_row1 * GROUP + (rd ^ (64 * s))),
-                           *(lds_x4)(st + a_row1 * GROUP + (rd ^ (64 * s) ^ 16)));
-        }
-#pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            if (b < active_b) {
-                const lds_bytes bt = st + STAGE_A + (th * 128 + b * 32) * GROUP;
-                const intx8 B0 = join(*(lds_x4)(bt + rd), *(lds_x4)(bt + (rd ^ 16)));
-                const intx8 B1 = join(*(lds_x4)(bt + (rd ^ 64)), *(lds_x4)(bt + (rd ^ 64 ^ 16)));
-                const float bs = *(const __attribute__((address_space(3))) float*)(
-                    st + STAGE_A + STAGE_B + (th * 128 + b * 32 + r32) * 4);
-                floatx16 p0 = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(A[0][0], B0, floatx16{0}, 0, 0,
-                                                                               0, 0, 0, 0);
-                floatx16 p1 = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(A[1][0], B0, floatx16{0}, 0, 0,
-                                                                               0, 0, 0, 0);
-                p0 = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(A[0][1], B1, p0, 0, 0, 0, 0, 0, 0);
-                p1 = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(A[1][1], B1, p1, 0, 0, 0, 0, 0, 0);
-                acc[0][b] += p0 * (bs * w0);
-                acc[1][b] += p1 * (bs * w1);
+        for (int b = 0; b < NB; ++b) {
+            p0 = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(A[0][0], B[0], floatx16{0}, 0, 0, 0, 0, 0, 0);
+            p0 = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(A[0][1], B[1], p0, 0, 0, 0, 0, 0, 0);
+            if (b > 0) {
+                acc[1][b - 1] += p1 * s1_prev;  // runs under the two MFMAs above
+                asm volatile("" : "+v"(acc[1][b - 1]));
             }
+            loads(2 * b);
+            __builtin_amdgcn_sched_barrier(0);
+            p1 = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(A[1][0], B[0], floatx16{0}, 0, 0, 0, 0, 0, 0);
+            p1 = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(A[1][1], B[1], p1, 0, 0, 0, 0, 0, 0);
+            const float s0 = bs * w0;
+            s1_prev = bs * w1;
+            if (b + 1 < NB) {
+                read_b(b + 1);
+                bs = read_bs(b + 1);
+            }
+            acc[0][b] += p0 * s0;  // p0 is complete by the time the MFMAs above are in
+            asm volatile("" : "+v"(acc[0][b]));
+            loads(2 * b + 1);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        asm volatile("" ::: "memory");
+        acc[1][NB > 0 ? NB - 1 : 0] += p1 * s1_prev;
+    };
+
+    PHASE_TIMING_BEGIN();
+    issue_scales(0, 0);
+#pragma unroll
+    for (int i = 4; i < 8; ++i) issue_load(0, i, 0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) issue_load(0, i, 0);
+    if (KB > 1) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) issue_load(1, i, 1);
     }
+    PHASE_MARK(0);  // prologue
+    // the K loop exists once per value of NB, so that the accumulators live in one place per copy
+    auto k_loop = [&](auto nb_tag) {
+        for (int kb = 0; kb < KB; ++kb) {
+            if (KB > 1) {
+                // everything but the 4 weight loads of block kb+1 (past the end: harmless ones)
+                __builtin_amdgcn_s_waitcnt((4 & 15) | ((4 >> 4) << 14) | (7 << 4) | (15 << 8));
+                asm volatile("" ::: "memory");
+            } else {
+                wait_all_loads();
+            }
+            PHASE_MARK(1);  // wait for this wavefront's own loads
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            PHASE_MARK(2);  // wait for the other wavefronts
+            block(nb_tag, kb, kb + 1 < KB ? kb + 1 : 0, kb + 2 < KB ? kb + 2 : 0);
+            asm volatile("" ::: "memory");
+            PHASE_MARK(4);  // operand reads, MFMAs, promotion, loads of later blocks
+        }
+    };
+    switch (active_b) {
+        case 4: k_loop(IntConstant<4>{}); break;
+        case 3: k_loop(IntConstant<3>{}); break;
+        case 2: k_loop(IntConstant<2>{}); break;
+        case 1: k_loop(IntConstant<1>{}); break;
+        default: k_loop(IntConstant<0>{}); break;
+    }
+    wait_all_loads();
     __syncthreads();  // the stages are free: reuse them for the epilogue exchange
+    PHASE_MARK(5);
 
     // result layout: register i of acc[a][b] is row 8*(i/4) + 4*half + i%4 of A tile a, pair
     // th*128 + b*32 + r32 of the tile
@@ -307,6 +429,8 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
             }
         }
     }
+    PHASE_MARK(6);  // epilogue
+    PHASE_TIMING_END(wave, lane);
 }
 
 }  // namespace
