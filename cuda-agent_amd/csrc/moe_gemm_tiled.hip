@@ -16,7 +16,9 @@
 //   the two A tiles of a wavefront stay in registers for the whole block while the four B
 //   tiles stream through: 24 KB of LDS reads per wavefront and block, 16 MFMAs.
 //
-// LDS slot of 16-byte chunk c of row r: r*8 + (c ^ (r & 7)), conflict-free for the fill and
+// LDS slot of 16-byte chunk c of row r: r*8 + (c ^ ((r >> 1) & 7)) (a ds_read_b128 serves 16
+// consecutive lanes per cycle from 64 banks, i.e. two 128-byte rows per bank row, so the 8 rows of
+// equal parity among 16 consecutive rows must use 8 different chunks), conflict-free for the fill and
 // for both operand reads. For gate/up the 256 rows are 128 gate rows and the matching 128 up
 // rows, each wavefront holding 32 of either, so SiLU(gate)*up and the e4m3 requantisation of
 // the 128-column group happen in the epilogue without leaving the workgroup.
@@ -172,10 +174,13 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
 
     // ---- fill side -------------------------------------------------------------------------
     // instruction j of a region covers its rows 8j..8j+7; lane -> row 8j + lane/8, chunk
-    // (lane%8) ^ (lane/8). This wavefront issues instructions 4*wave .. 4*wave+3 of A and of B.
+    // (lane%8) ^ ((row >> 1) & 7). This wavefront issues instructions 4*wave .. 4*wave+3 of A and of B.
     const uint32_t ld_row = lane >> 3;
-    const uint32_t ld_chunk = (lane & 7) ^ ld_row;
-    const uint32_t ld_off = ld_row * (uint32_t)K + 16 * ld_chunk;
+    // the row's swizzle term ((row >> 1) & 7) is (ld_row >> 1) for even and 4 ^ (ld_row >> 1) for
+    // odd instructions of a wavefront (its first instruction index is a multiple of 4)
+    const uint32_t ld_chunk_even = (lane & 7) ^ (ld_row >> 1);
+    const uint32_t ld_off_even = ld_row * (uint32_t)K + 16 * ld_chunk_even;
+    const uint32_t ld_off_odd = ld_row * (uint32_t)K + 16 * (ld_chunk_even ^ 4);
     const uint8_t* a_src[4];
     uint32_t b_off[4];  // byte offset of this lane's activation row and chunk (the buffers are < 4 GB)
 #pragma unroll
@@ -188,7 +193,7 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
         int p = (4 * wave + i) * 8 + (int)ld_row;
         p = begin + (p < cnt ? p : cnt - 1);  // rows past the tile's end repeat the last one
         const int arow = GATE_UP ? sorted_pairs[p] / top_k : p;
-        b_off[i] = (uint32_t)arow * (uint32_t)K + 16 * ld_chunk;
+        b_off[i] = (uint32_t)arow * (uint32_t)K + 16 * (ld_chunk_even ^ (4 * (i & 1)));
     }
     const float* s_src = as_t + begin;  // + kb*scale_stride; 256 floats, the tail is padding
     const float* ws0;
@@ -206,7 +211,7 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
     auto issue_load = [&](int kb, int i, int slot_parity) {
         const uint32_t st = stage_base + (slot_parity & 1) * STAGE_BYTES;
         if (i < 4) {
-            dma16(a_src[i] + (size_t)kb * GROUP, ld_off, st + (4 * wave + i) * 1024);
+            dma16(a_src[i] + (size_t)kb * GROUP, (i & 1) ? ld_off_odd : ld_off_even, st + (4 * wave + i) * 1024);
         } else {
             dma16(a_q + (size_t)kb * GROUP, b_off[i - 4], st + STAGE_A + (4 * wave + i - 4) * 1024);
         }
@@ -218,7 +223,7 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
 
     // ---- read side -------------------------------------------------------------------------
     // operand of k-step s, 16-byte piece j: chunk 4s + 2*half + j of row r32 (+32*tile)
-    const uint32_t rd = (r32 * 8 + ((2 * half) ^ (r32 & 7))) * 16;
+    const uint32_t rd = (r32 * 8 + ((2 * half) ^ ((r32 >> 1) & 7))) * 16;
     const uint32_t a_row0 = GATE_UP ? rg * 32 : rg * 64;        // A tile 0 of this wavefront
     const uint32_t a_row1 = GATE_UP ? 128 + rg * 32 : rg * 64 + 32;
     const lds_bytes stage_ptr = (lds_bytes)s_stage;
@@ -275,20 +280,25 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
             read_b(0);
             bs = read_bs(0);
         }
-        issue_scales(kb1, kb + 1);
-#pragma unroll
-        for (int i = 4; i < 8; ++i) issue_load(kb1, i, kb + 1);
         // every wavefront holds its A operands: the weight half of this stage may be refilled
         __builtin_amdgcn_s_waitcnt((63 & 15) | ((63 >> 4) << 14) | (7 << 4) | (0 << 8));  // lgkmcnt(0)
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        constexpr int PER_SLOT = NB >= 2 ? 1 : NB == 1 ? 2 : 4;  // weight loads per MFMA pair
+        // load sequence of the block: pair scales and activations of block kb+1 (load numbers
+        // 0..3), then the weights of block kb+2 (4..7), spread over the MFMA pairs
+        auto load_number = [&](int n) {
+            if (n == 0) issue_scales(kb1, kb + 1);
+            if (n < 4) issue_load(kb1, 4 + n, kb + 1);
+            else issue_load(kb2, n - 4, kb);
+        };
+        constexpr int PER_SLOT = NB >= 3 ? 2 : NB == 2 ? 2 : NB == 1 ? 4 : 8;
         auto loads = [&](int slot) {
 #pragma unroll
             for (int j = 0; j < PER_SLOT; ++j) {
-                const int i = slot * PER_SLOT + j;
-                if (i < 4) issue_load(kb2, i, kb);
+                // NB >= 3: activations two per slot (slots 0, 1), weights one per slot (slots 2..5)
+                const int n = NB >= 3 ? (slot < 2 ? 2 * slot + j : (j == 0 ? slot + 2 : 8)) : slot * PER_SLOT + j;
+                if (n < 8) load_number(n);
             }
         };
         if (NB == 0) {
