@@ -51,9 +51,14 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
 
-// position of 16-byte chunk `chunk` of row `row` inside a tile (in 16-byte units)
+// position of 16-byte chunk `chunk` of row `row` inside a tile (in 16-byte units). A row is 1152
+// bytes = 4.5 x 256, so two consecutive rows share a row of the 64 LDS banks like rows of 128
+// bytes would; a ds_read_b128 serves 16 consecutive lanes per cycle, so among 16 consecutive
+// tile rows the 8 of equal parity must use 8 different chunk positions: the swizzle term is
+// (row >> 1) & 7 (with row & 7 the K operand reads ran at 2/3 of the conflict-free rate).
+__device__ __forceinline__ int row_swizzle(int row) { return (row >> 1) & 7; }
 __device__ __forceinline__ int swizzled_slot(int row, int chunk) {
-    return row * ROW_CHUNKS + ((chunk & ~7) | ((chunk ^ row) & 7));
+    return row * ROW_CHUNKS + ((chunk & ~7) | ((chunk ^ row_swizzle(row)) & 7));
 }
 
 // One wavefront's share of a tile: with NW wavefronts each owns 32/NW consecutive rows, fetched by
@@ -77,7 +82,7 @@ struct TileLoader {
         const int slot = inst * 64 + l;
         const int row = slot / ROW_CHUNKS;
         const int pos = slot - row * ROW_CHUNKS;
-        const int chunk = (pos & ~7) | ((pos ^ row) & 7);
+        const int chunk = (pos & ~7) | ((pos ^ row_swizzle(row)) & 7);
         const int key = s_idx_tile[row];
         const char* src = kv_b + (size_t)(key < 0 ? 0 : key) * ROW_BYTES + chunk * 16;
         // Each lane's 16 bytes land at lds_base + lane*16 (M0 carries the wavefront's base).
@@ -125,7 +130,8 @@ constexpr float FRAME_SLACK = 0.f;
 struct LaneOffsets {
     uint32_t qk[4];  // K operand of k-step ks: qk[ks & 3] + (ks >> 2) * 128
     uint32_t pv[2];  // V^T operand of dv tile t, k-step ks, half-read rr:
-                     //   pv[t & 1] + (16*ks + 8*rr) * ROW_BYTES + (t >> 1) * 128
+                     //   (pv[t & 1] ^ 64*rr) + (16*ks + 8*rr) * ROW_BYTES + (t >> 1) * 128
+                     // (8 rows further down the swizzle term has bit 2 flipped)
 };
 
 __device__ __forceinline__ LaneOffsets make_lane_offsets(int lane) {
@@ -134,7 +140,7 @@ __device__ __forceinline__ LaneOffsets make_lane_offsets(int lane) {
     const int half = lane >> 5;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-        o.qk[c] = r32 * ROW_BYTES + (((2 * c + half) ^ r32) & 7) * 16;
+        o.qk[c] = r32 * ROW_BYTES + (((2 * c + half) ^ row_swizzle(r32)) & 7) * 16;
     }
     const int g2 = (lane >> 4) & 1;
     const int s16 = lane & 15;
@@ -142,7 +148,7 @@ __device__ __forceinline__ LaneOffsets make_lane_offsets(int lane) {
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
         const int chunk = 4 * u + 2 * g2 + ((s16 & 3) >> 1);
-        o.pv[u] = row * ROW_BYTES + ((chunk ^ row) & 7) * 16 + 8 * (s16 & 1);
+        o.pv[u] = row * ROW_BYTES + ((chunk ^ row_swizzle(row)) & 7) * 16 + 8 * (s16 & 1);
     }
     return o;
 }
@@ -264,7 +270,7 @@ __device__ __forceinline__ void process_tile(const uint4* tile, const int* s_idx
 #pragma unroll
         for (int rr = 0; rr < 2; ++rr) {
             dst[rr] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (lds_s4)(base + off.pv[t & 1] + (16 * ks + 8 * rr) * ROW_BYTES + (t >> 1) * 128));
+                (lds_s4)(base + (off.pv[t & 1] ^ (64 * rr)) + (16 * ks + 8 * rr) * ROW_BYTES + (t >> 1) * 128));
         }
     };
 #pragma unroll
@@ -508,7 +514,7 @@ __device__ __forceinline__ void gather_prepare(uint32_t (&off)[GATHER_INSTR], co
 #pragma unroll
     for (int i = 0; i < GATHER_INSTR; ++i) {
         const int key = *reinterpret_cast<const int*>(keys + (e[i] >> 16));
-        off[i] = (uint32_t)key * (uint32_t)ROW_BYTES + (e[i] & 0xffffu);
+        off[i] = (uint32_t)key * (uint32_t)ROW_BYTES + ((e[i] & 0xffffu) ^ ((quarter & 1) << 6));
         if (has_padding && key < 0) off[i] = GATHER_MASKED;
     }
 }
@@ -570,9 +576,9 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
     }
     if (tid == 0) s_first_masked_tile = n_tiles;
     for (int c = tid; c < GATHER_TAB; c += 512) {
-        const int row = c / ROW_CHUNKS;  // 0..7; the tile row is 8*quarter + row, same low 3 bits
-        const int pos = c - row * ROW_CHUNKS;
-        const int chunk = (pos & ~7) | ((pos ^ row) & 7);
+        const int row = c / ROW_CHUNKS;  // 0..7; the tile row is 8*quarter + row: for odd quarters the
+        const int pos = c - row * ROW_CHUNKS;  // swizzle term has bit 2 flipped (gather_prepare)
+        const int chunk = (pos & ~7) | ((pos ^ row_swizzle(row)) & 7);
         s_gather_tab[c] = ((uint32_t)(4 * row) << 16) | (uint32_t)(chunk * 16);
     }
     __syncthreads();
@@ -628,7 +634,7 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
     SoftmaxState st{-INFINITY, 0.f};
     const LaneOffsets off = make_lane_offsets(lane);
     // K operand of local step l: qk_l[l & 1] + (l >> 1) * 128
-    // V^T operand of local dv tile tl: pv_l[tl & 1] + (16*ks + 8*rr) * ROW_BYTES + (tl >> 1) * 128
+    // V^T operand of local dv tile tl: (pv_l[tl & 1] ^ 64*rr) + (16*ks + 8*rr) * ROW_BYTES + (tl >> 1) * 128
     const uint32_t qk_l[2] = {dh ? off.qk[2] : off.qk[0], dh ? off.qk[3] : off.qk[1]};
     const uint32_t pv_l[2] = {off.pv[0] + 512u * dh, off.pv[1] + 512u * dh};
     floatx4* my_xchg = &s_xchg[wave][0];
@@ -766,7 +772,7 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
 #pragma unroll
                 for (int rr = 0; rr < 2; ++rr) {
                     dst[j][rr] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (lds_s4)(base + pv_l[tl & 1] + (16 * ks + 8 * rr) * ROW_BYTES + (tl >> 1) * 128));
+                        (lds_s4)(base + (pv_l[tl & 1] ^ (64 * rr)) + (16 * ks + 8 * rr) * ROW_BYTES + (tl >> 1) * 128));
                 }
             }
         };
