@@ -377,10 +377,14 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
     PHASE_MARK(5);
 
     // result layout: register i of acc[a][b] is row 8*(i/4) + 4*half + i%4 of A tile a, pair
-    // th*128 + b*32 + r32 of the tile
+    // th*128 + b*32 + r32 of the tile. In that layout a store instruction would touch 32 or 64
+    // different output rows with 4 to 32 bytes each, so both epilogues transpose through LDS and
+    // write every output row as one contiguous run.
     if (GATE_UP) {
-        float* s_amax = reinterpret_cast<float*>(s_stage);  // [4 row groups][256 pairs]
-        float amax[4];
+        float* s_amax = reinterpret_cast<float*>(s_stage);                      // [4 row groups][256 pairs]
+        constexpr int CODE_ROW = GROUP + 16;                                    // bytes per pair row of codes
+        uint8_t* s_codes = s_stage + 4 * TILE_PAIRS * sizeof(float);            // [256 pairs][CODE_ROW]
+        static_assert(4 * TILE_PAIRS * sizeof(float) + TILE_PAIRS * CODE_ROW <= 2 * STAGE_BYTES, "epilogue LDS");
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
             float m = 0.f;
@@ -391,50 +395,74 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
                 m = fmaxf(m, fabsf(v));
             }
             m = fmaxf(m, __shfl_xor(m, 32));
-            amax[b] = m;
             if (half == 0) s_amax[rg * TILE_PAIRS + th * 128 + b * 32 + r32] = m;
         }
         __syncthreads();
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
             const int pl = th * 128 + b * 32 + r32;
-            if (pl < cnt) {
-                const float m = fmaxf(fmaxf(s_amax[pl], s_amax[TILE_PAIRS + pl]),
-                                      fmaxf(s_amax[2 * TILE_PAIRS + pl], s_amax[3 * TILE_PAIRS + pl]));
-                const float scale = fmaxf(m, AMAX_FLOOR) * INV_E4M3_MAX;
+            const float m = fmaxf(fmaxf(s_amax[pl], s_amax[TILE_PAIRS + pl]),
+                                  fmaxf(s_amax[2 * TILE_PAIRS + pl], s_amax[3 * TILE_PAIRS + pl]));
+            const float scale = fmaxf(m, AMAX_FLOOR) * INV_E4M3_MAX;
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd) {
+                float q[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    q[r] = fminf(fmaxf(acc[0][b][4 * qd + r] / scale, -E4M3_MAX), E4M3_MAX);
+                }
+                int packed = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], 0, false);
+                packed = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], packed, true);
+                *reinterpret_cast<int*>(s_codes + pl * CODE_ROW + rg * 32 + 8 * qd + 4 * half) = packed;
+            }
+            if (rg == 0 && half == 0 && pl < cnt) {
                 const size_t pos = (size_t)begin + pl;
+                h_s[pos * (inter / GROUP) + rb] = scale;
+                hs_t[(size_t)rb * scale_stride + pos] = scale;
+            }
+        }
+        __syncthreads();
+        // 8 lanes write the 128 codes of one pair: 8 pairs per instruction, 4 instructions per wavefront
 #pragma unroll
-                for (int qd = 0; qd < 4; ++qd) {
-                    float q[4];
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        q[r] = fminf(fmaxf(acc[0][b][4 * qd + r] / scale, -E4M3_MAX), E4M3_MAX);
-                    }
-                    int packed = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], 0, false);
-                    packed = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], packed, true);
-                    *reinterpret_cast<int*>(h_q + pos * inter + rb * GROUP + rg * 32 + 8 * qd + 4 * half) =
-                        packed;
-                }
-                if (rg == 0 && half == 0) {
-                    h_s[pos * (inter / GROUP) + rb] = scale;
-                    hs_t[(size_t)rb * scale_stride + pos] = scale;
-                }
+        for (int it = 0; it < 4; ++it) {
+            const int pl = (wave * 4 + it) * 8 + (lane >> 3);
+            if (pl < cnt) {
+                const intx4 v = *reinterpret_cast<const intx4*>(s_codes + pl * CODE_ROW + (lane & 7) * 16);
+                *reinterpret_cast<intx4*>(h_q + ((size_t)begin + pl) * inter + rb * GROUP + (lane & 7) * 16) = v;
             }
         }
     } else {
+        // two passes of 128 pairs: the wavefronts of one pair half put their 64 x 128 results into
+        // LDS as [pair][256 rows], then all 8 wavefronts write whole 1 KB rows
+        constexpr int Y_ROW = TILE_ROWS + 4;  // floats per staged pair row (16 bytes of padding)
+        static_assert(128 * Y_ROW * sizeof(float) <= 2 * STAGE_BYTES, "epilogue LDS");
+        float* s_y = reinterpret_cast<float*>(s_stage);
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            const int pl = th * 128 + b * 32 + r32;
-            if (pl < cnt) {
-                float* dst = y + ((size_t)begin + pl) * n_rows + rb * TILE_ROWS + rg * 64 + 4 * half;
+        for (int pass = 0; pass < 2; ++pass) {
+            if (pass == 1) __syncthreads();
+            if (th == pass) {
 #pragma unroll
-                for (int a = 0; a < 2; ++a) {
+                for (int b = 0; b < 4; ++b) {
+                    float* dst = s_y + (b * 32 + r32) * Y_ROW + rg * 64 + 4 * half;
 #pragma unroll
-                    for (int qd = 0; qd < 4; ++qd) {
-                        *reinterpret_cast<floatx4*>(dst + a * 32 + 8 * qd) =
-                            floatx4{acc[a][b][4 * qd], acc[a][b][4 * qd + 1], acc[a][b][4 * qd + 2],
-                                    acc[a][b][4 * qd + 3]};
+                    for (int a = 0; a < 2; ++a) {
+#pragma unroll
+                        for (int qd = 0; qd < 4; ++qd) {
+                            *reinterpret_cast<floatx4*>(dst + a * 32 + 8 * qd) =
+                                floatx4{acc[a][b][4 * qd], acc[a][b][4 * qd + 1], acc[a][b][4 * qd + 2],
+                                        acc[a][b][4 * qd + 3]};
+                        }
                     }
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int it = 0; it < 16; ++it) {
+                const int pr = wave * 16 + it;  // pair within this half
+                const int pl = pass * 128 + pr;
+                if (pl < cnt) {
+                    const floatx4 v = *reinterpret_cast<const floatx4*>(s_y + pr * Y_ROW + lane * 4);
+                    *reinterpret_cast<floatx4*>(y + ((size_t)begin + pl) * n_rows + rb * TILE_ROWS + lane * 4) = v;
                 }
             }
         }
