@@ -34,10 +34,10 @@ FP8_PEAK_TFLOPS = 5033.0
 METRIC = "GB/s & % HBM peak (GDN/MoE/MLA decode); fp8 TFLOP/s % MFMA peak (MoE prefill)"
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled
-# by the same counters read on a plain 512 MiB copy kernel (FETCH_SIZE x 1.99984, WRITE_SIZE x 1,
+# by the same counters read on a plain 512 MiB copy kernel (FETCH_SIZE x 1.99981, WRITE_SIZE x 1,
 # both in KiB); the counter summary is profiles/all_workloads_hbm_traffic_pmc.md.
 # None = not measured.
-MEASURED_TRAFFIC = {'gdn': 1085986734, 'moe_decode': 6664742582, 'mla': 277476469, 'moe_prefill': 11202932427}
+MEASURED_TRAFFIC = {'gdn': 1085972770, 'moe_decode': 6664643628, 'mla': 256686692, 'moe_prefill': 11270026834}
 
 
 def timed_launches(torch, launch, steps, warmup):
