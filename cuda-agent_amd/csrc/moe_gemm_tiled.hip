@@ -86,14 +86,21 @@ __device__ __forceinline__ void dma16_ptr(const void* lane_ptr, uint32_t lds_bas
 __global__ __launch_bounds__(1024) void moe_tile_start_kernel(const int* __restrict__ expert_offsets,
                                                               int* __restrict__ tile_start,
                                                               int n_experts) {
-    if (threadIdx.x == 0) {
-        int running = 0;
-        for (int e = 0; e < n_experts; ++e) {
-            tile_start[e] = running;
-            running += (expert_offsets[e + 1] - expert_offsets[e] + TILE_PAIRS - 1) / TILE_PAIRS;
-        }
-        tile_start[n_experts] = running;
+    __shared__ int s_tiles[1024 + 1];
+    const int t = threadIdx.x;
+    const int mine = t < n_experts ? (expert_offsets[t + 1] - expert_offsets[t] + TILE_PAIRS - 1) / TILE_PAIRS : 0;
+    int v = mine;
+    if (t < n_experts) s_tiles[t] = v;
+    __syncthreads();
+    for (int d = 1; d < n_experts; d <<= 1) {
+        const int add = (t >= d && t < n_experts) ? s_tiles[t - d] : 0;
+        __syncthreads();
+        v += add;
+        if (t < n_experts) s_tiles[t] = v;
+        __syncthreads();
     }
+    if (t < n_experts) tile_start[t] = v - mine;
+    if (t == n_experts - 1) tile_start[n_experts] = v;
 }
 
 // xs_t[kb][pos] = x_s[token of sorted position pos][kb]

@@ -84,60 +84,157 @@ __global__ __launch_bounds__(256) void moe_hist_kernel(const int* __restrict__ i
     }
 }
 
+// Exclusive prefix sum of s[0..n) in place (n <= 1024, blockDim.x == 1024); s[n] = total.
+__device__ __forceinline__ void block_exclusive_scan(int* s, int n) {
+    const int t = threadIdx.x;
+    const int mine = t < n ? s[t] : 0;
+    int v = mine;
+    __syncthreads();
+    for (int d = 1; d < n; d <<= 1) {
+        const int add = (t >= d && t < n) ? s[t - d] : 0;
+        __syncthreads();
+        v += add;
+        if (t < n) s[t] = v;
+        __syncthreads();
+    }
+    if (t < n) s[t] = v - mine;
+    if (t == n - 1) s[n] = v;
+    __syncthreads();
+}
+
 // In place: chunk_hist[chunk][e] becomes the first sorted position of expert e's pairs from
-// that chunk; expert_offsets[e] the first position of the expert. One workgroup.
+// that chunk; expert_offsets[e] the first position of the expert. One workgroup; the loads of a
+// column are issued in independent batches (a read-modify-write loop over the chunks is one
+// memory latency per chunk).
 __global__ __launch_bounds__(1024) void moe_scan_kernel(int* __restrict__ chunk_hist,
                                                         int* __restrict__ expert_offsets,
                                                         int chunks, int n_experts) {
-    extern __shared__ int s_count[];  // [n_experts]
-    for (int e = threadIdx.x; e < n_experts; e += 1024) {
-        int running = 0;
-        for (int c = 0; c < chunks; ++c) {
-            const int v = chunk_hist[(size_t)c * n_experts + e];
-            chunk_hist[(size_t)c * n_experts + e] = running;
-            running += v;
+    __shared__ int s_count[1024 + 1];
+    constexpr int BATCH = 8;
+    const int e = threadIdx.x;
+    int total = 0;
+    if (e < n_experts) {
+        for (int c0 = 0; c0 < chunks; c0 += BATCH) {
+            int v[BATCH];
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) {
+                v[j] = c0 + j < chunks ? chunk_hist[(size_t)(c0 + j) * n_experts + e] : 0;
+            }
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) total += v[j];
         }
-        s_count[e] = running;
+        s_count[e] = total;
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        int running = 0;
-        for (int e = 0; e < n_experts; ++e) {
-            const int v = s_count[e];
-            s_count[e] = running;
-            expert_offsets[e] = running;
-            running += v;
+    block_exclusive_scan(s_count, n_experts);
+    if (e < n_experts) {
+        int running = s_count[e];
+        expert_offsets[e] = running;
+        for (int c0 = 0; c0 < chunks; c0 += BATCH) {
+            int v[BATCH];
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) {
+                v[j] = c0 + j < chunks ? chunk_hist[(size_t)(c0 + j) * n_experts + e] : 0;
+            }
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) {
+                if (c0 + j < chunks) chunk_hist[(size_t)(c0 + j) * n_experts + e] = running;
+                running += v[j];
+            }
         }
-        expert_offsets[n_experts] = running;
     }
-    __syncthreads();
-    for (int e = threadIdx.x; e < n_experts; e += 1024) {
-        const int base = s_count[e];
-        for (int c = 0; c < chunks; ++c) chunk_hist[(size_t)c * n_experts + e] += base;
+    if (e == 0) expert_offsets[n_experts] = s_count[n_experts];
+}
+
+// rank of this lane's pair among the pairs of the same 64-pair group with the same expert
+// (`earlier`), and whether a later lane of the group has the same expert
+__device__ __forceinline__ void group_rank(int e, int lane, int& earlier, bool& later) {
+    earlier = 0;
+    later = false;
+#pragma unroll 8
+    for (int k = 0; k < 64; ++k) {
+        const int ek = __builtin_amdgcn_readlane(e, k);
+        earlier += (ek == e && k < lane) ? 1 : 0;
+        later = later || (ek == e && k > lane);
     }
 }
 
-// Lane e walks the chunk's pairs in flat order; every pair of expert e takes e's next position.
-__global__ __launch_bounds__(256) void moe_scatter_kernel(const int* __restrict__ ids,
-                                                          const int* __restrict__ chunk_base,
-                                                          int* __restrict__ sorted_pairs,
-                                                          int* __restrict__ pair_pos, int pairs,
-                                                          int pairs_per_chunk, int n_experts) {
-    extern __shared__ int s_ids[];  // [pairs_per_chunk]
+// Stable scatter of one chunk in three parallel phases. The chunk's pairs are taken in groups of
+// 64 in flat order: (1) one wavefront per group ranks its pairs among equal experts of the group
+// and leaves the group's count per expert in LDS; (2) one lane per expert turns the counts into
+// first positions, group after group, starting from the chunk's first position for that expert;
+// (3) every pair is written to (first position of its expert in its group) + (its rank).
+// LDS: [groups][n_experts] counts + [groups*64] ranks.
+__global__ __launch_bounds__(1024) void moe_scatter_kernel(const int* __restrict__ ids,
+                                                           const int* __restrict__ chunk_base,
+                                                           int* __restrict__ sorted_pairs,
+                                                           int* __restrict__ pair_pos, int pairs,
+                                                           int pairs_per_chunk, int n_experts) {
+    extern __shared__ int s_mem[];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
     const int begin = blockIdx.x * pairs_per_chunk;
     int count = pairs - begin;
     if (count > pairs_per_chunk) count = pairs_per_chunk;
-    for (int i = threadIdx.x; i < count; i += 256) s_ids[i] = ids[begin + i];
+    const int groups = (count + 63) / 64;
+    int* s_first = s_mem;                       // [groups][n_experts]
+    int* s_rank = s_mem + groups * n_experts;   // [groups * 64]
+    for (int i = threadIdx.x; i < groups * n_experts; i += 1024) s_first[i] = 0;
     __syncthreads();
-    for (int e = threadIdx.x; e < n_experts; e += 256) {
-        int next = chunk_base[(size_t)blockIdx.x * n_experts + e];
-        for (int i = 0; i < count; ++i) {
-            if (s_ids[i] == e) {
-                sorted_pairs[next] = begin + i;
-                pair_pos[begin + i] = next;
-                ++next;
-            }
+    for (int g = wave; g < groups; g += 16) {
+        const int i = g * 64 + lane;
+        const int e = i < count ? ids[begin + i] : -1 - lane;  // lanes past the end match nobody
+        int earlier;
+        bool later;
+        group_rank(e, lane, earlier, later);
+        s_rank[i] = earlier;
+        if (i < count && !later) s_first[g * n_experts + e] = earlier + 1;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < n_experts; e += 1024) {
+        int running = chunk_base[(size_t)blockIdx.x * n_experts + e];
+        for (int g = 0; g < groups; ++g) {
+            const int v = s_first[g * n_experts + e];
+            s_first[g * n_experts + e] = running;
+            running += v;
         }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < count; i += 1024) {
+        const int pos = s_first[(i >> 6) * n_experts + ids[begin + i]] + s_rank[i];
+        sorted_pairs[pos] = begin + i;
+        pair_pos[begin + i] = pos;
+    }
+}
+
+// The same order with one wavefront per chunk and n_experts ints of LDS, for chunks whose group
+// table would not fit: a pair's position is (next free position of its expert) + (its rank in the
+// group); the last lane of every expert present then advances that expert's position.
+__global__ __launch_bounds__(64) void moe_scatter_serial_kernel(const int* __restrict__ ids,
+                                                                const int* __restrict__ chunk_base,
+                                                                int* __restrict__ sorted_pairs,
+                                                                int* __restrict__ pair_pos, int pairs,
+                                                                int pairs_per_chunk, int n_experts) {
+    extern __shared__ int s_next[];  // [n_experts]
+    const int lane = threadIdx.x;
+    const int begin = blockIdx.x * pairs_per_chunk;
+    int count = pairs - begin;
+    if (count > pairs_per_chunk) count = pairs_per_chunk;
+    for (int e = lane; e < n_experts; e += 64) s_next[e] = chunk_base[(size_t)blockIdx.x * n_experts + e];
+    __syncthreads();
+    for (int g = 0; g < count; g += 64) {
+        const int i = g + lane;
+        const int e = i < count ? ids[begin + i] : -1 - lane;
+        int earlier;
+        bool later;
+        group_rank(e, lane, earlier, later);
+        if (i < count) {
+            const int pos = s_next[e] + earlier;
+            sorted_pairs[pos] = begin + i;
+            pair_pos[begin + i] = pos;
+            if (!later) s_next[e] = pos + 1;
+        }
+        __syncthreads();
     }
 }
 
@@ -258,7 +355,7 @@ extern "C" void moe_sort_launcher(int* sorted_pairs, int* pair_pos, int* expert_
                                   int top_k, int config, hipStream_t stream) {
     (void)config;
     if (tokens <= 0) return;
-    if (n_experts <= 0 || n_experts > 4096 || top_k <= 0 || top_k > 64) {
+    if (n_experts <= 0 || n_experts > 1024 || top_k <= 0 || top_k > 64) {
         caa::set_status(CAA_UNSUPPORTED_SHAPE);
         return;
     }
@@ -271,10 +368,15 @@ extern "C" void moe_sort_launcher(int* sorted_pairs, int* pair_pos, int* expert_
     const int chunks = (tokens + moe::SORT_CHUNK_TOKENS - 1) / moe::SORT_CHUNK_TOKENS;
     moe_hist_kernel<<<chunks, 256, n_experts * sizeof(int), stream>>>(ids, chunk_scratch, pairs,
                                                                      pairs_per_chunk, n_experts);
-    moe_scan_kernel<<<1, 1024, n_experts * sizeof(int), stream>>>(chunk_scratch, expert_offsets, chunks,
-                                                                 n_experts);
-    moe_scatter_kernel<<<chunks, 256, pairs_per_chunk * sizeof(int), stream>>>(
-        ids, chunk_scratch, sorted_pairs, pair_pos, pairs, pairs_per_chunk, n_experts);
+    moe_scan_kernel<<<1, 1024, 0, stream>>>(chunk_scratch, expert_offsets, chunks, n_experts);
+    const size_t group_table = ((size_t)(pairs_per_chunk / 64) * n_experts + pairs_per_chunk) * sizeof(int);
+    if (group_table <= 64 * 1024) {
+        moe_scatter_kernel<<<chunks, 1024, group_table, stream>>>(ids, chunk_scratch, sorted_pairs, pair_pos,
+                                                                  pairs, pairs_per_chunk, n_experts);
+    } else {
+        moe_scatter_serial_kernel<<<chunks, 64, n_experts * sizeof(int), stream>>>(
+            ids, chunk_scratch, sorted_pairs, pair_pos, pairs, pairs_per_chunk, n_experts);
+    }
 }
 
 extern "C" void moe_route_sort_launcher(int* ids, float* weights, int* sorted_pairs, int* pair_pos,

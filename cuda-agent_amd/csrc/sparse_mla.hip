@@ -885,6 +885,7 @@ int pick_splits(int batch, int head_groups, int topk, int config) {
 
 extern "C" int sparse_mla_decode_num_splits(int batch, int n_heads, int topk, int config) {
     if (batch <= 0 || n_heads <= 0 || topk <= 0) return 0;
+    if (config >= 1000) config -= 1000;  // 1000 + n: n splits on the one-wavefront-per-head-group kernel
     const int head_groups = n_heads <= 128 ? 1 : n_heads / 128;
     return pick_splits(batch, head_groups, topk, config);
 }
@@ -924,7 +925,7 @@ extern "C" void sparse_mla_decode_launcher(void* out, const void* q, const void*
         caa::set_status(CAA_BAD_ARGUMENT);
         return;
     }
-    if (workspace_bytes < sparse_mla_decode_workspace_bytes(batch, n_heads, topk, config % 1000)) {
+    if (workspace_bytes < sparse_mla_decode_workspace_bytes(batch, n_heads, topk, config)) {
         caa::set_status(CAA_WORKSPACE_TOO_SMALL);
         return;
     }

@@ -84,7 +84,9 @@ void gdn_decode_launcher(float* o, float* state, const void* q, const void* k, c
  * 16-byte aligned.
  * config: 0 chooses the number of key splits so that about one workgroup per CU is resident;
  * n > 0 forces n splits (raised if a split would exceed 2048 rows, lowered to the number of
- * 32-row tiles). */
+ * 32-row tiles). 1000 + n: as n, on the kernel with one wavefront per 32 heads, which multiples of
+ * 128 heads otherwise use only when a request's cache block is 4 GB or larger (the default kernel
+ * for them addresses the block with 32-bit offsets). */
 void sparse_mla_decode_launcher(void* out, const void* q, const void* kv, const int* idx,
                                 void* workspace, size_t workspace_bytes, int batch, int n_heads,
                                 int n_kv_rows, int topk, int d_qk, int d_v, float sm_scale,

@@ -113,6 +113,17 @@ def test_split_counts_agree(capi, dev):
         assert mla.rel_rms_error(o, outs[0]) <= TOL
 
 
+def test_one_wavefront_per_head_group_kernel_for_128_heads(capi, dev):
+    # config 1000 + n selects the kernel that caches of 4 GB and more per request fall back to
+    gen = torch.Generator().manual_seed(14)
+    q, kv, idx = (t.to(dev) for t in mla.mla_make_inputs(2, 128, 900, 300, generator=gen))
+    padded = torch.cat([idx[:, :100], torch.full((2, 20), -1, dtype=torch.int32, device=dev), idx[:, 100:]],
+                       dim=1).contiguous()
+    ref = oracle_on_gpu(q, kv, padded)
+    for config in (1000, 1001, 1003):
+        check(capi, q, kv, padded, config, ref)
+
+
 def test_large_scores_do_not_overflow(capi, dev):
     gen = torch.Generator().manual_seed(13)
     q, kv, idx = (t.to(dev) for t in mla.mla_make_inputs(1, 128, 300, 200, generator=gen))
