@@ -57,11 +57,21 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
     const int t = blockIdx.x;
     for (int c = (blockIdx.y * 256 + threadIdx.x) * 4; c < hidden; c += gridDim.y * 1024) {
         floatx4 acc = {0.f, 0.f, 0.f, 0.f};
-        for (int k = 0; k < top_k; ++k) {
-            const int pos = pair_pos[(size_t)t * top_k + k];
-            const float w = weights[(size_t)t * top_k + k];
-            const floatx4 v = *reinterpret_cast<const floatx4*>(y + (size_t)pos * hidden + c);
-            acc += v * w;
+        // four rows are fetched at a time (independent loads); the sum still runs in ascending k
+        for (int k0 = 0; k0 < top_k; k0 += 4) {
+            floatx4 v[4];
+            float w[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int k = k0 + j < top_k ? k0 + j : k0;
+                const int pos = pair_pos[(size_t)t * top_k + k];
+                w[j] = weights[(size_t)t * top_k + k];
+                v[j] = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(y + (size_t)pos * hidden + c));
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (k0 + j < top_k) acc += v[j] * w[j];
+            }
         }
         OUT* dst = out + (size_t)t * hidden + c;
         if constexpr (sizeof(OUT) == 4) {
