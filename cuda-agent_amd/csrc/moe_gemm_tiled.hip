@@ -120,7 +120,9 @@ __global__ __launch_bounds__(256) void moe_gather_scales_kernel(const float* __r
 // cycles it spends in each phase of the K loop and leaves them in g_phase_cycles.
 #ifdef MOE_PHASE_TIMING
 __device__ unsigned long long g_phase_cycles[8][8];
-#define PHASE_TIMING_BEGIN() unsigned long long phase_t0 = __builtin_readcyclecounter(), phase_acc[8] = {}
+#define PHASE_TIMING_BEGIN()                                                              \
+    unsigned long long phase_t0 = __builtin_readcyclecounter(), phase_acc[8] = {};        \
+    const unsigned long long phase_wall0 = wall_clock64(), phase_core0 = phase_t0
 #define PHASE_MARK(n)                                                      \
     {                                                                      \
         const unsigned long long phase_now = __builtin_readcyclecounter(); \
@@ -129,7 +131,9 @@ __device__ unsigned long long g_phase_cycles[8][8];
     }
 #define PHASE_TIMING_END(wave, lane)                                        \
     if (blockIdx.x == 0 && (lane) == 0) {                                   \
-        for (int i = 0; i < 8; ++i) g_phase_cycles[wave][i] = phase_acc[i]; \
+        for (int i = 0; i < 7; ++i) g_phase_cycles[wave][i] = phase_acc[i]; \
+        /* core clock in kHz over the workgroup's life: the wall clock counts at 100 MHz */ \
+        g_phase_cycles[wave][7] = (__builtin_readcyclecounter() - phase_core0) * 100000ull / (wall_clock64() - phase_wall0); \
     }
 #else
 #define PHASE_TIMING_BEGIN()
