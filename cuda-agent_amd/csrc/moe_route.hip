@@ -22,6 +22,12 @@ __device__ __forceinline__ unsigned long long rank_key(float logit, int id) {
     return ((unsigned long long)u << 32) | (unsigned)(0x7fffffff - id);  // lower id wins a tie
 }
 
+// the logit a key was made from (-0 comes back as +0, which has the same sigmoid)
+__device__ __forceinline__ float key_logit(unsigned long long key) {
+    const unsigned u = (unsigned)(key >> 32);
+    return __uint_as_float((u & 0x80000000u) ? (u & 0x7fffffffu) : ~u);
+}
+
 template <int PER_LANE>
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits,
                                                         int* __restrict__ ids,
@@ -53,7 +59,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
         for (int j = 0; j < PER_LANE; ++j) {
             if (j * 64 + lane == id) key[j] = 0ull;  // taken
         }
-        const float logit = logits[(size_t)t * n_experts + id];
+        const float logit = key_logit(best);
         const float score = 1.f / (1.f + expf(-logit));
         total += score;
         if (lane == k) {
@@ -276,7 +282,7 @@ __global__ __launch_bounds__(1024) void moe_route_sort_small_kernel(
             for (int j = 0; j < PER_LANE; ++j) {
                 if (j * 64 + lane == id) key[j] = 0ull;
             }
-            const float score = 1.f / (1.f + expf(-logits[(size_t)t * n_experts + id]));
+            const float score = 1.f / (1.f + expf(-key_logit(best)));
             total += score;
             if (lane == k) {
                 my_score = score;
@@ -298,16 +304,7 @@ __global__ __launch_bounds__(1024) void moe_route_sort_small_kernel(
         for (int i = 0; i < p; ++i) rank += s_ids[i] == mine;
     }
     __syncthreads();
-    if (threadIdx.x == 0) {  // exclusive scan of the counts, in place
-        int running = 0;
-        for (int e = 0; e < n_experts; ++e) {
-            const int c = s_count[e];
-            s_count[e] = running;
-            running += c;
-        }
-        s_count[n_experts] = running;
-    }
-    __syncthreads();
+    block_exclusive_scan(s_count, n_experts);  // in place; s_count[n_experts] = number of pairs
     for (int e = threadIdx.x; e <= n_experts; e += 1024) expert_offsets[e] = s_count[e];
     if (p < pairs) {
         const int pos = s_count[mine] + rank;
