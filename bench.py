@@ -40,8 +40,26 @@ METRIC = "GB/s & % HBM peak (GDN/MoE/MLA decode); fp8 TFLOP/s % MFMA peak (MoE p
 MEASURED_TRAFFIC = {'gdn': 1085972770, 'moe_decode': 6664643628, 'mla': 256686692, 'moe_prefill': 11270026834}
 
 
+SETTLE_SECONDS = 0.05
+
+
 def timed_launches(torch, launch, steps, warmup):
-    """Average device time of one launch in seconds, HIP events on the current (launch) stream."""
+    """Average device time of one launch in seconds, HIP events on the current (launch) stream.
+
+    Before the `warmup` untimed steps the same launch is repeated for about SETTLE_SECONDS, untimed:
+    the first few milliseconds of work after the inputs were generated run at lower clocks (the first
+    workload of a process measured 5-6 % low without it).
+    """
+    launch(0)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    n = 0
+    while time.perf_counter() - t0 < SETTLE_SECONDS:
+        launch(n)
+        n += 1
+        if n % 8 == 0:
+            torch.cuda.synchronize()
+    torch.cuda.synchronize()
     for i in range(warmup):
         launch(i)
     torch.cuda.synchronize()
@@ -267,7 +285,8 @@ def main():
         "metric": METRIC, "value": head['value'], "unit": head['unit'], "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": head['ms_per_step'], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": head['dtype'], "data": "synthetic",
-        "config": {"workload": head['workload']},
+        "config": {"workload": head['workload'],
+                   "settle": f"{SETTLE_SECONDS} s of untimed launches before the warm-up steps of every workload"},
         "roofline": head['roofline'],
     }
     if 'cpu_baseline' in head:
