@@ -37,7 +37,7 @@ METRIC = "GB/s & % HBM peak (GDN/MoE/MLA decode); fp8 TFLOP/s % MFMA peak (MoE p
 # by the same counters read on a plain 512 MiB copy kernel (FETCH_SIZE x 1.99981, WRITE_SIZE x 1,
 # both in KiB); the counter summary is profiles/all_workloads_hbm_traffic_pmc.md.
 # None = not measured.
-MEASURED_TRAFFIC = {'gdn': 1085972770, 'moe_decode': 6664643628, 'mla': 256686692, 'moe_prefill': 11270026834}
+MEASURED_TRAFFIC = {'gdn': 1085972770, 'moe_decode': 6664643628, 'mla': 256686692, 'moe_prefill': 11230161000}
 
 
 SETTLE_SECONDS = 0.05
@@ -117,6 +117,36 @@ def bench_gdn(torch, capi, dev, steps, warmup, cpu_baseline):
         res['cpu_baseline'] = dict(value=work / csec / 1e9, unit="GB/s", cores=cores, kind="port",
                                    sample="the full configs[1] step (eager PyTorch oracle, state in place), "
                                           "1 warm-up + up to 5 timed steps")
+    return res
+
+
+def bench_gdn_fused(torch, capi, dev, steps, warmup, cpu_baseline):
+    """configs[1] sizes through the launcher that also does the caller's pre-step (L2 normalisation of
+    q and k, decay and write gates): same bytes, the gate inputs a, b take the place of g, beta."""
+    from oracle import gdn
+    B, Hv, Hqk = 256, 32, 16
+    gen = torch.Generator().manual_seed(20256)
+    host = gdn.gdn_make_raw_inputs(B, Hv, Hqk, qkv_dtype=torch.bfloat16, generator=gen)
+    q, k, v, a, b, a_log, dt_bias, state0 = (t.to(dev) for t in host)
+    sets = [(torch.empty(B, Hv, 128, device=dev), state0.clone()) for _ in range(3)]
+    sec = timed_launches(
+        torch, lambda i: capi.gdn_decode_fused_launch(*sets[i % 3], q, k, v, a, b, a_log, dt_bias), steps, warmup)
+    work = 2 * B * Hv * 128 * 128 * 4 + 2 * B * Hqk * 128 * 2 + B * Hv * 128 * 2 + 2 * B * Hv * 4 + B * Hv * 128 * 4 \
+        + 2 * Hv * 4
+    res = dict(
+        workload="configs[1] sizes with the pre-step fused (raw q/k normalised in the kernel, gates from a, b, "
+                 "A_log, dt_bias), seed 20256",
+        value=work / sec / 1e9, unit="GB/s", ms_per_step=sec * 1e3, dtype="f32", kernel="gdn_decode_kernel<fused>",
+        roofline=dict(bound="hbm", achieved=work / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
+                      frac=work / sec / 1e9 / HBM_PEAK_GBS, traffic=None),
+        algorithmic_bytes=work)
+    if cpu_baseline:
+        cores = len(os.sched_getaffinity(0))
+        torch.set_num_threads(cores)
+        csec = cpu_time(lambda: gdn.gdn_decode_fused_step(*host))
+        res['cpu_baseline'] = dict(value=work / csec / 1e9, unit="GB/s", cores=cores, kind="port",
+                                   sample="the full step (eager PyTorch oracle, state in place), 1 warm-up + up to "
+                                          "5 timed steps")
     return res
 
 
@@ -237,7 +267,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=20)
     ap.add_argument('--warmup', type=int, default=5)
-    ap.add_argument('--workloads', default='gdn,moe_decode,mla,moe_prefill')
+    ap.add_argument('--workloads', default='gdn,gdn_fused,moe_decode,mla,moe_prefill')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run 3 plain device copies of 536 870 912 bytes (a kernel of known traffic, '
@@ -268,6 +298,8 @@ def main():
     for name in wanted:
         if name == 'gdn':
             results[name] = bench_gdn(torch, capi, dev, args.steps, args.warmup, cpu)
+        elif name == 'gdn_fused':
+            results[name] = bench_gdn_fused(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'mla':
             results[name] = bench_mla(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'moe_decode':

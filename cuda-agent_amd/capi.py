@@ -20,6 +20,8 @@ SIGNATURES = {
     'axpby_launcher': (None, [_P, _P, _P, c_float, c_int, c_int, _P]),
     'gdn_decode_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int,
                                    c_int, c_int, _P]),
+    'gdn_decode_fused_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int,
+                                         c_int, c_int, c_int, _P]),
     'sparse_mla_decode_launcher': (None, [_P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int,
                                           c_int, c_int, c_float, c_int, c_int, _P]),
     'sparse_mla_decode_num_splits': (c_int, [c_int, c_int, c_int, c_int]),
@@ -120,6 +122,28 @@ def gdn_decode_launch(o, state, q, k, v, g, beta, config=0, stream=None):
                                   _ptr(beta), B, Hv, Hqk, dk, dv,
                                   0 if q.dtype == torch.float32 else 1, config, _stream(stream))
     check_status('gdn_decode_launcher')
+    return o, state
+
+
+def gdn_decode_fused_launch(o, state, q, k, v, a, b, a_log, dt_bias, config=0, stream=None):
+    """One decode step from unnormalised q/k and the gate inputs (see the header); ``state`` is
+    updated in place and ``o`` written."""
+    import torch
+    _device_contiguous(o=o, state=state, q=q, k=k, v=v, a=a, b=b, a_log=a_log, dt_bias=dt_bias)
+    B, Hv, dk, dv = state.shape
+    Hqk = q.shape[1]
+    _require(all(t.dtype == torch.float32 for t in (state, o, a, b, a_log, dt_bias)),
+             'gdn_decode_fused: o, state, a, b, a_log, dt_bias must be fp32')
+    _require(q.dtype == k.dtype == v.dtype and q.dtype in (torch.float32, torch.bfloat16),
+             'gdn_decode_fused: q, k, v must share dtype fp32 or bf16')
+    _require(tuple(q.shape) == (B, Hqk, dk) and tuple(k.shape) == (B, Hqk, dk), 'gdn_decode_fused: q/k shape')
+    _require(tuple(v.shape) == (B, Hv, dv) and tuple(o.shape) == (B, Hv, dv), 'gdn_decode_fused: v/o shape')
+    _require(tuple(a.shape) == (B, Hv) and tuple(b.shape) == (B, Hv), 'gdn_decode_fused: a/b shape')
+    _require(tuple(a_log.shape) == (Hv,) and tuple(dt_bias.shape) == (Hv,), 'gdn_decode_fused: a_log/dt_bias shape')
+    library().gdn_decode_fused_launcher(_ptr(o), _ptr(state), _ptr(q), _ptr(k), _ptr(v), _ptr(a), _ptr(b),
+                                        _ptr(a_log), _ptr(dt_bias), B, Hv, Hqk, dk, dv,
+                                        0 if q.dtype == torch.float32 else 1, config, _stream(stream))
+    check_status('gdn_decode_fused_launcher')
     return o, state
 
 

@@ -57,11 +57,15 @@ __device__ __forceinline__ void store_state(float* p, float4 x, bool nt) {
     }
 }
 
-template <typename T, int COLS, int THREADS, int NT>
+// FUSED: q and k arrive unnormalised and are scaled by rsqrt(sum x^2 + 1e-6) here (the factors are
+// applied to the reductions, not to the 128 values); `g` and `beta` are then the per-request
+// gate inputs a and b, and g = exp(-exp(a_log[h]) * softplus(a + dt_bias[h])), beta = sigmoid(b).
+template <typename T, int COLS, int THREADS, int NT, bool FUSED = false>
 __global__ __launch_bounds__(THREADS) void gdn_decode_kernel(
     float* __restrict__ o, float* __restrict__ state, const T* __restrict__ q,
     const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ g,
-    const float* __restrict__ beta, int n_v_heads, int n_qk_heads, float scale) {
+    const float* __restrict__ beta, int n_v_heads, int n_qk_heads, float scale,
+    const float* __restrict__ a_log = nullptr, const float* __restrict__ dt_bias = nullptr) {
     constexpr int WAVES = THREADS / 64;
     constexpr int CG = COLS / 4;            // float4 column groups per row segment
     constexpr int RPP = THREADS / CG;       // rows covered by one pass of the workgroup
@@ -72,6 +76,9 @@ __global__ __launch_bounds__(THREADS) void gdn_decode_kernel(
     __shared__ float s_q[DK];
     __shared__ float s_k[DK];
     __shared__ float s_kq[WAVES];
+    __shared__ float s_qq[WAVES];  // FUSED: sums of squares
+    __shared__ float s_kk[WAVES];
+    __shared__ float s_gate[2];    // FUSED: g and beta of the unit, computed by one lane
     __shared__ float4 s_red[2][WAVES][CG];
 
     const int tid = threadIdx.x;
@@ -88,19 +95,42 @@ __global__ __launch_bounds__(THREADS) void gdn_decode_kernel(
 
     float* S = state + (size_t)unit * (DK * DV) + tile * COLS + cg * 4;
 
-    // Issue the whole state tile's loads first; everything below overlaps their latency.
+    // The small vectors are requested first and the state tile right behind them: loads return in
+    // order, so q, k and the gates can be reduced while the 64 KB of state are still on their way
+    // (the other way round, the two wavefronts that hold q and k would wait for their state rows
+    // before they could start the k.q reduction everybody else then waits for).
+    const T* qh = q + ((size_t)b * n_qk_heads + hq) * DK;
+    const T* kh = k + ((size_t)b * n_qk_heads + hq) * DK;
+    // FUSED with at least 6 wavefronts: lanes DK..2DK-1 read q and lanes 2DK..3DK-1 read k a second
+    // time and reduce the sums of squares, in parallel with the k.q reduction of lanes 0..DK-1
+    constexpr bool SPLIT_NORMS = FUSED && THREADS >= 3 * DK;
+    float qv = 0.f, kv = 0.f;
+    if (tid < DK) {
+        qv = to_f32(qh[tid]);
+        kv = to_f32(kh[tid]);
+    } else if (SPLIT_NORMS && tid < 2 * DK) {
+        qv = to_f32(qh[tid - DK]);
+    } else if (SPLIT_NORMS && tid < 3 * DK) {
+        kv = to_f32(kh[tid - 2 * DK]);
+    }
+    float gate_a = 0.f, gate_b = 0.f, gate_alog = 0.f, gate_dt = 0.f;
+    if (!FUSED || tid == THREADS - 1) {
+        gate_a = g[unit];
+        gate_b = beta[unit];
+        if (FUSED) {
+            gate_alog = a_log[hv];
+            gate_dt = dt_bias[hv];
+        }
+    }
+
     float4 s[NP];
 #pragma unroll
     for (int m = 0; m < NP; ++m) {
         s[m] = load_state(S + (size_t)(r0 + m * RPP) * DV, NT == 1 || NT == 2);
     }
 
-    const T* qh = q + ((size_t)b * n_qk_heads + hq) * DK;
-    const T* kh = k + ((size_t)b * n_qk_heads + hq) * DK;
     float kq_part = 0.f;
     if (tid < DK) {
-        const float qv = to_f32(qh[tid]);
-        const float kv = to_f32(kh[tid]);
         s_q[tid] = qv;
         s_k[tid] = kv;
         kq_part = qv * kv;
@@ -110,13 +140,46 @@ __global__ __launch_bounds__(THREADS) void gdn_decode_kernel(
         for (int off = 32; off >= 1; off >>= 1) kq_part += __shfl_xor(kq_part, off);
         if (lane == 0) s_kq[wave] = kq_part;
     }
+    if (FUSED && (SPLIT_NORMS ? (tid >= DK && tid < 3 * DK) : tid < DK)) {
+        float qq_part = qv * qv, kk_part = kv * kv;  // (one of them is 0 when the work is split)
+        if (SPLIT_NORMS) {
+            float part = qq_part + kk_part;
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) part += __shfl_xor(part, off);
+            if (lane == 0) (tid < 2 * DK ? s_qq : s_kk)[wave & 1] = part;
+        } else {
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) {
+                qq_part += __shfl_xor(qq_part, off);
+                kk_part += __shfl_xor(kk_part, off);
+            }
+            if (lane == 0) {
+                s_qq[wave] = qq_part;
+                s_kk[wave] = kk_part;
+            }
+        }
+    }
     const float4 vj = [&] {
         const T* vh = v + (size_t)unit * DV + tile * COLS + cg * 4;
         return make_float4(to_f32(vh[0]), to_f32(vh[1]), to_f32(vh[2]), to_f32(vh[3]));
     }();
-    const float gh = g[unit];
-    const float bh = beta[unit];
+    float gh = gate_a, bh = gate_b;
+    if (FUSED && tid == THREADS - 1) {  // one lane of a wavefront that has no q/k work
+        // hardware exp/log (about 1 ulp of fp32 on the ranges met here); log(1 + e^x) instead of
+        // log1p loses at most 1e-7 absolute, far below the fp32 noise of the 128-term sums
+        const float x = gate_a + gate_dt;
+        const float softplus = x > 20.f ? x : __logf(1.f + __expf(x));
+        s_gate[0] = __expf(-__expf(gate_alog) * softplus);
+        s_gate[1] = 1.f / (1.f + __expf(-gate_b));
+    }
     __syncthreads();
+    float inv_q = 1.f, inv_k = 1.f;
+    if (FUSED) {
+        gh = s_gate[0];
+        bh = s_gate[1];
+        inv_q = rsqrtf(s_qq[0] + s_qq[1] + 1e-6f);
+        inv_k = rsqrtf(s_kk[0] + s_kk[1] + 1e-6f);
+    }
 
     // a = S0^T k and c = S0^T q over this lane's rows
     float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -125,8 +188,8 @@ __global__ __launch_bounds__(THREADS) void gdn_decode_kernel(
 #pragma unroll
     for (int m = 0; m < NP; ++m) {
         const int r = r0 + m * RPP;
-        kr[m] = s_k[r];
-        const float qr = s_q[r];
+        kr[m] = s_k[r] * inv_k;
+        const float qr = s_q[r] * inv_q;
         a.x += s[m].x * kr[m]; a.y += s[m].y * kr[m]; a.z += s[m].z * kr[m]; a.w += s[m].w * kr[m];
         c.x += s[m].x * qr;    c.y += s[m].y * qr;    c.z += s[m].z * qr;    c.w += s[m].w * qr;
     }
@@ -152,7 +215,7 @@ __global__ __launch_bounds__(THREADS) void gdn_decode_kernel(
         a.x += aw.x; a.y += aw.y; a.z += aw.z; a.w += aw.w;
         c.x += cw.x; c.y += cw.y; c.z += cw.z; c.w += cw.w;
     }
-    const float kq = s_kq[0] + s_kq[1];
+    const float kq = (s_kq[0] + s_kq[1]) * (inv_q * inv_k);
 
     float4 d;
     d.x = bh * (vj.x - gh * a.x);
@@ -182,26 +245,33 @@ __global__ __launch_bounds__(THREADS) void gdn_decode_kernel(
 
 template <typename T, int COLS, int THREADS, int NT>
 void launch_variant(float* o, float* state, const T* q, const T* k, const T* v, const float* g,
-                    const float* beta, int units, int n_v_heads, int n_qk_heads,
-                    hipStream_t stream) {
+                    const float* beta, const float* a_log, const float* dt_bias, int units,
+                    int n_v_heads, int n_qk_heads, hipStream_t stream) {
     const float scale = 0.08838834764831845f;  // 128^-1/2
-    gdn_decode_kernel<T, COLS, THREADS, NT><<<dim3(units * (DV / COLS)), THREADS, 0, stream>>>(
-        o, state, q, k, v, g, beta, n_v_heads, n_qk_heads, scale);
+    const dim3 grid(units * (DV / COLS));
+    if (a_log) {
+        gdn_decode_kernel<T, COLS, THREADS, NT, true><<<grid, THREADS, 0, stream>>>(
+            o, state, q, k, v, g, beta, n_v_heads, n_qk_heads, scale, a_log, dt_bias);
+    } else {
+        gdn_decode_kernel<T, COLS, THREADS, NT, false><<<grid, THREADS, 0, stream>>>(
+            o, state, q, k, v, g, beta, n_v_heads, n_qk_heads, scale);
+    }
 }
 
+// a_log != nullptr selects the fused form (g and beta are then the gate inputs a and b)
 template <typename T>
 void launch(float* o, float* state, const void* q, const void* k, const void* v, const float* g,
-            const float* beta, int batch, int n_v_heads, int n_qk_heads, int config,
-            hipStream_t stream) {
+            const float* beta, const float* a_log, const float* dt_bias, int batch, int n_v_heads,
+            int n_qk_heads, int config, hipStream_t stream) {
     const int units = batch * n_v_heads;
     const T* qt = static_cast<const T*>(q);
     const T* kt = static_cast<const T*>(k);
     const T* vt = static_cast<const T*>(v);
     if (config <= 0 || config > 12) config = units >= 2048 ? 9 : 12;  // few heads: smaller tiles
-#define GDN_VARIANT(id, cols, threads, nt)                                                     \
-    case id:                                                                                   \
-        launch_variant<T, cols, threads, nt>(o, state, qt, kt, vt, g, beta, units, n_v_heads,  \
-                                             n_qk_heads, stream);                              \
+#define GDN_VARIANT(id, cols, threads, nt)                                                         \
+    case id:                                                                                       \
+        launch_variant<T, cols, threads, nt>(o, state, qt, kt, vt, g, beta, a_log, dt_bias, units, \
+                                             n_v_heads, n_qk_heads, stream);                       \
         break;
     switch (config) {
         GDN_VARIANT(1, 128, 256, 0)
@@ -220,6 +290,11 @@ void launch(float* o, float* state, const void* q, const void* k, const void* v,
 #undef GDN_VARIANT
 }
 
+bool gdn_shape_ok(int batch, int n_v_heads, int n_qk_heads, int dk, int dv, int qkv_dtype) {
+    return dk == DK && dv == DV && n_qk_heads > 0 && n_v_heads % n_qk_heads == 0 &&
+           (qkv_dtype == 0 || qkv_dtype == 1) && (long)batch * n_v_heads * 4 <= 0x7fffffffL;
+}
+
 }  // namespace
 
 // o      [batch, n_v_heads, 128] fp32, written
@@ -234,8 +309,7 @@ extern "C" void gdn_decode_launcher(float* o, float* state, const void* q, const
                                     int n_v_heads, int n_qk_heads, int dk, int dv, int qkv_dtype,
                                     int config, hipStream_t stream) {
     if (batch <= 0 || n_v_heads <= 0) return;
-    if (dk != DK || dv != DV || n_qk_heads <= 0 || n_v_heads % n_qk_heads != 0 ||
-        (qkv_dtype != 0 && qkv_dtype != 1) || (long)batch * n_v_heads * 4 > 0x7fffffffL) {
+    if (!gdn_shape_ok(batch, n_v_heads, n_qk_heads, dk, dv, qkv_dtype)) {
         caa::set_status(CAA_UNSUPPORTED_SHAPE);
         return;
     }
@@ -245,9 +319,38 @@ extern "C" void gdn_decode_launcher(float* o, float* state, const void* q, const
         return;
     }
     if (qkv_dtype == 0) {
-        launch<float>(o, state, q, k, v, g, beta, batch, n_v_heads, n_qk_heads, config, stream);
+        launch<float>(o, state, q, k, v, g, beta, nullptr, nullptr, batch, n_v_heads, n_qk_heads, config,
+                      stream);
     } else {
-        launch<__hip_bfloat16>(o, state, q, k, v, g, beta, batch, n_v_heads, n_qk_heads, config,
+        launch<__hip_bfloat16>(o, state, q, k, v, g, beta, nullptr, nullptr, batch, n_v_heads, n_qk_heads,
+                               config, stream);
+    }
+}
+
+// The same step with the caller's pre-step fused in: q and k [batch, n_qk_heads, 128] arrive
+// unnormalised and are scaled by rsqrt(sum x^2 + 1e-6); a, b [batch, n_v_heads] fp32 are the gate
+// inputs, a_log, dt_bias [n_v_heads] fp32 the per-head parameters:
+//   g = exp(-exp(a_log[h]) * softplus(a + dt_bias[h])),  beta = sigmoid(b).
+// Everything else as gdn_decode_launcher.
+extern "C" void gdn_decode_fused_launcher(float* o, float* state, const void* q, const void* k,
+                                          const void* v, const float* a, const float* b,
+                                          const float* a_log, const float* dt_bias, int batch,
+                                          int n_v_heads, int n_qk_heads, int dk, int dv,
+                                          int qkv_dtype, int config, hipStream_t stream) {
+    if (batch <= 0 || n_v_heads <= 0) return;
+    if (!gdn_shape_ok(batch, n_v_heads, n_qk_heads, dk, dv, qkv_dtype)) {
+        caa::set_status(CAA_UNSUPPORTED_SHAPE);
+        return;
+    }
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(o) | reinterpret_cast<uintptr_t>(state);
+    if (!o || !state || !q || !k || !v || !a || !b || !a_log || !dt_bias || (bits & 15u) != 0) {
+        caa::set_status(CAA_BAD_ARGUMENT);
+        return;
+    }
+    if (qkv_dtype == 0) {
+        launch<float>(o, state, q, k, v, a, b, a_log, dt_bias, batch, n_v_heads, n_qk_heads, config, stream);
+    } else {
+        launch<__hip_bfloat16>(o, state, q, k, v, a, b, a_log, dt_bias, batch, n_v_heads, n_qk_heads, config,
                                stream);
     }
 }

@@ -68,6 +68,18 @@ void gdn_decode_launcher(float* o, float* state, const void* q, const void* k, c
                          int n_qk_heads, int dk, int dv, int qkv_dtype, int config,
                          hipStream_t stream);
 
+/* The same step with the step in front of it fused in (the caller of the path in Qwen3-Next-style
+ * layers; same launcher pattern, agent_workdir/kernels/axpby.cu:12-20): q and k arrive
+ * unnormalised and are scaled by rsqrt(sum x^2 + 1e-6) per head inside the kernel, and the gates
+ * are computed from
+ *   a, b [batch, n_v_heads] fp32 (per-request gate inputs), a_log, dt_bias [n_v_heads] fp32:
+ *   g = exp(-exp(a_log[h]) * softplus(a + dt_bias[h])),  beta = sigmoid(b).
+ * Everything else as gdn_decode_launcher. */
+void gdn_decode_fused_launcher(float* o, float* state, const void* q, const void* k, const void* v,
+                               const float* a, const float* b, const float* a_log,
+                               const float* dt_bias, int batch, int n_v_heads, int n_qk_heads,
+                               int dk, int dv, int qkv_dtype, int config, hipStream_t stream);
+
 /* Sparse-MLA decode attention (workload config 3 of the benchmark definition; launcher
  * pattern agent_workdir/kernels/axpby.cu:12-20). Per request every head attends to the rows
  * of that request's latent cache listed in idx:

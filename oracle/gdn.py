@@ -17,6 +17,13 @@ Pinned by (tests/test_oracle_gdn.py):
     GQA equals the ungrouped rule fed the repeated q/k heads;
   * a golden fixture written from an independent third-party implementation of the same
     recurrence (tests/golden/make_gdn_golden.py).
+
+``gdn_prestep`` / ``gdn_decode_fused_step`` add the caller's step in front of the recurrence
+(L2 normalisation of q and k, decay and write-strength gates). Pinned by: unit norm and scale
+invariance of the normalised vectors, ``softplus``/``sigmoid``/``rsqrt`` library routines against
+float64 closed forms, limits (a_log -> -inf gives g = 1), and a second golden fixture from the same
+third-party function called with its in-kernel L2 normalisation switched on and the gate computed by
+library calls (tests/golden/make_gdn_golden.py, ``gdn_fused_golden.npz``).
 """
 
 import math
@@ -42,6 +49,51 @@ def gdn_decode_step(q, k, v, g, beta, state):
     state.add_(kf[:, :, :, None] * delta[:, :, None, :])
     o = torch.einsum('bhij,bhi->bhj', state, qf) * (dk ** -0.5)
     return o, state
+
+
+L2NORM_EPS = 1e-6
+
+
+def gdn_prestep(q_raw, k_raw, a, b, a_log, dt_bias):
+    """The step in front of the recurrence in Qwen3-Next-style layers (the caller of the path;
+    restated from the third-party ``transformers`` layer, models/qwen3_next/modeling_qwen3_next.py:
+    ``l2norm`` at :368-371 and the gate lines ``beta = b.sigmoid()``,
+    ``g = -A_log.exp() * softplus(a + dt_bias)`` at :659-661, whose recurrent kernel then uses
+    ``exp(g)``). Returns ``(q, k, g, beta)`` in the form ``gdn_decode_step`` takes: q, k fp32
+    L2-normalised as ``x * rsqrt(sum(x*x) + 1e-6)``, ``g = exp(-exp(a_log) * softplus(a + dt_bias))``
+    the decay itself, ``beta = sigmoid(b)``.
+
+    q_raw, k_raw: [B, Hqk, dk] (bf16 or fp32); a, b: [B, Hv]; a_log, dt_bias: [Hv] fp32.
+    """
+    qf, kf = q_raw.float(), k_raw.float()
+    qn = qf * torch.rsqrt((qf * qf).sum(-1, keepdim=True) + L2NORM_EPS)
+    kn = kf * torch.rsqrt((kf * kf).sum(-1, keepdim=True) + L2NORM_EPS)
+    g = torch.exp(-torch.exp(a_log.float()) * torch.nn.functional.softplus(a.float() + dt_bias.float()))
+    beta = torch.sigmoid(b.float())
+    return qn, kn, g, beta
+
+
+def gdn_decode_fused_step(q_raw, k_raw, v, a, b, a_log, dt_bias, state):
+    """Pre-step followed by the recurrence; mutates ``state`` and returns ``(o, state)``."""
+    qn, kn, g, beta = gdn_prestep(q_raw, k_raw, a, b, a_log, dt_bias)
+    return gdn_decode_step(qn, kn, v, g, beta, state)
+
+
+def gdn_make_raw_inputs(batch, n_v_heads, n_qk_heads, dk=128, dv=128, qkv_dtype=torch.float32,
+                        generator=None):
+    """Inputs of the fused form: q, k ~ N(0, 1) * U(0.5, 2) per head (not normalised), v ~ N(0,1),
+    a, b ~ N(0,1), a_log ~ U(-1, 1), dt_bias ~ U(-1, 1), state ~ N(0, 0.02).
+    Returns ``[q_raw, k_raw, v, a, b, a_log, dt_bias, state]``."""
+    gen = generator
+    q = torch.randn(batch, n_qk_heads, dk, generator=gen) * (0.5 + 1.5 * torch.rand(batch, n_qk_heads, 1, generator=gen))
+    k = torch.randn(batch, n_qk_heads, dk, generator=gen) * (0.5 + 1.5 * torch.rand(batch, n_qk_heads, 1, generator=gen))
+    v = torch.randn(batch, n_v_heads, dv, generator=gen)
+    a = torch.randn(batch, n_v_heads, generator=gen)
+    b = torch.randn(batch, n_v_heads, generator=gen)
+    a_log = 2 * torch.rand(n_v_heads, generator=gen) - 1
+    dt_bias = 2 * torch.rand(n_v_heads, generator=gen) - 1
+    state = 0.02 * torch.randn(batch, n_v_heads, dk, dv, generator=gen)
+    return [q.to(qkv_dtype), k.to(qkv_dtype), v.to(qkv_dtype), a, b, a_log, dt_bias, state]
 
 
 def gdn_decode_loops_f64(q, k, v, g, beta, state):

@@ -33,6 +33,22 @@ def main():
                         state=state.numpy(), o=o[:, 0].numpy(), new_state=new_state.numpy())
     print('wrote', out, out.stat().st_size, 'bytes')
 
+    # fused form: raw q/k normalised inside the third-party function (use_qk_l2norm_in_kernel),
+    # log-decay from library calls as in that layer's forward
+    from oracle.gdn import gdn_make_raw_inputs
+    gen = torch.Generator().manual_seed(434343)
+    qr, kr, v, a, b, a_log, dt_bias, state = gdn_make_raw_inputs(B, Hv, Hqk, dk, dv, generator=gen)
+    log_g = -a_log.float().exp() * torch.nn.functional.softplus(a.float() + dt_bias)
+    o, new_state = fn(
+        qr.repeat_interleave(rep, 1)[:, None], kr.repeat_interleave(rep, 1)[:, None], v[:, None],
+        log_g[:, None], b.sigmoid()[:, None], initial_state=state.clone(), output_final_state=True,
+        use_qk_l2norm_in_kernel=True)
+    out = Path(__file__).with_name('gdn_fused_golden.npz')
+    np.savez_compressed(out, q=qr.numpy(), k=kr.numpy(), v=v.numpy(), a=a.numpy(), b=b.numpy(),
+                        a_log=a_log.numpy(), dt_bias=dt_bias.numpy(), state=state.numpy(),
+                        o=o[:, 0].numpy(), new_state=new_state.numpy())
+    print('wrote', out, out.stat().st_size, 'bytes')
+
 
 if __name__ == '__main__':
     main()

@@ -145,3 +145,54 @@ def test_workspace_rejects_bad_inputs(dev):
         "print('ok')\n")
     out = subprocess.run([sys.executable, '-c', code], cwd=ws, capture_output=True, text=True, timeout=300)
     assert out.returncode == 0 and 'ok' in out.stdout, out.stdout + out.stderr
+
+
+# ---- fused pre-step (L2 normalisation of q/k and gates inside the kernel) -------------------------
+
+FUSED_GOLDEN = Path(__file__).parent / 'golden' / 'gdn_fused_golden.npz'
+
+
+def run_fused(capi, dev, ins, config=0):
+    qr, kr, v, a, b, a_log, dt_bias, state = (t.to(dev) for t in ins)
+    o = torch.full((state.shape[0], state.shape[1], state.shape[3]), float('nan'), device=dev)
+    capi.gdn_decode_fused_launch(o, state, qr, kr, v, a, b, a_log, dt_bias, config=config)
+    torch.cuda.synchronize()
+    return o.cpu(), state.cpu()
+
+
+@pytest.mark.parametrize('config', [0, 1, 3, 9])
+@pytest.mark.parametrize('shape', [(1, 16, 16, torch.float32), (3, 8, 4, torch.bfloat16), (5, 4, 1, torch.float32)])
+def test_fused_matches_oracle(capi, dev, shape, config):
+    B, Hv, Hqk, dt = shape
+    gen = torch.Generator().manual_seed(300 + B)
+    ins = gdn.gdn_make_raw_inputs(B, Hv, Hqk, qkv_dtype=dt, generator=gen)
+    want_o, want_s = gdn.gdn_decode_fused_step(*ins[:7], ins[7].clone())
+    o, s = run_fused(capi, dev, ins, config)
+    assert gdn.gdn_close(o, want_o) and gdn.gdn_close(s, want_s)
+
+
+def test_fused_golden_fixture(capi, dev):
+    z = np.load(FUSED_GOLDEN)
+    ins = [torch.from_numpy(z[n]) for n in ('q', 'k', 'v', 'a', 'b', 'a_log', 'dt_bias', 'state')]
+    o, s = run_fused(capi, dev, ins)
+    assert gdn.gdn_close(o, torch.from_numpy(z['o'])) and gdn.gdn_close(s, torch.from_numpy(z['new_state']))
+
+
+def test_fused_equals_unfused_on_prestepped_inputs(capi, dev):
+    gen = torch.Generator().manual_seed(31)
+    ins = gdn.gdn_make_raw_inputs(4, 8, 4, generator=gen)
+    qn, kn, g, beta = gdn.gdn_prestep(*ins[:2], *ins[3:7])
+    o1, s1 = run_fused(capi, dev, ins)
+    o2, s2 = run_kernel(capi, dev, [qn, kn, ins[2], g, beta, ins[7]])
+    assert gdn.gdn_close(o1, o2) and gdn.gdn_close(s1, s2)
+
+
+def test_fused_full_workload_shape(capi, dev):
+    # configs[1] sizes; the pre-step must not cost bandwidth: compare with the unfused kernel's result
+    gen = torch.Generator().manual_seed(32)
+    ins = gdn.gdn_make_raw_inputs(256, 32, 16, qkv_dtype=torch.bfloat16, generator=gen)
+    qn, kn, g, beta = gdn.gdn_prestep(*ins[:2], *ins[3:7])
+    o1, s1 = run_fused(capi, dev, ins)
+    want_o, want_s = gdn.gdn_decode_step(qn.to(dev), kn.to(dev), ins[2].to(dev), g.to(dev), beta.to(dev),
+                                         ins[7].to(dev))
+    assert gdn.gdn_close(o1, want_o.cpu()) and gdn.gdn_close(s1, want_s.cpu())

@@ -104,3 +104,64 @@ def test_golden_fixture_from_third_party_recurrence():
     o, s = gdn.gdn_decode_step(*ins[:5], ins[5].clone())
     np.testing.assert_allclose(o.numpy(), z['o'], rtol=2e-5, atol=1e-7)
     np.testing.assert_allclose(s.numpy(), z['new_state'], rtol=2e-5, atol=1e-7)
+
+
+# ---- the caller's pre-step (L2 normalisation and gates) ------------------------------------------
+
+FUSED_GOLDEN = Path(__file__).parent / 'golden' / 'gdn_fused_golden.npz'
+
+
+def test_prestep_against_float64_closed_forms():
+    gen = torch.Generator().manual_seed(21)
+    qr, kr, v, a, b, a_log, dt_bias, _ = gdn.gdn_make_raw_inputs(3, 6, 3, 16, 8, generator=gen)
+    qn, kn, g, beta = gdn.gdn_prestep(qr, kr, a, b, a_log, dt_bias)
+    q64 = qr.double()
+    want_q = q64 / torch.sqrt((q64 * q64).sum(-1, keepdim=True) + 1e-6)
+    torch.testing.assert_close(qn.double(), want_q, rtol=1e-6, atol=1e-7)
+    x = (a.double() + dt_bias.double())
+    want_g = torch.exp(-torch.exp(a_log.double()) * torch.log1p(torch.exp(x)))   # softplus = log(1 + e^x)
+    torch.testing.assert_close(g.double(), want_g, rtol=1e-6, atol=1e-7)
+    torch.testing.assert_close(beta.double(), 1 / (1 + torch.exp(-b.double())), rtol=1e-6, atol=1e-7)
+    assert (g > 0).all() and (g < 1).all()
+
+
+def test_prestep_normalises_and_ignores_the_scale_of_q_and_k():
+    gen = torch.Generator().manual_seed(22)
+    qr, kr, v, a, b, a_log, dt_bias, state = gdn.gdn_make_raw_inputs(2, 4, 2, 32, 16, generator=gen)
+    qn, kn, _, _ = gdn.gdn_prestep(qr, kr, a, b, a_log, dt_bias)
+    torch.testing.assert_close(qn.norm(dim=-1), torch.ones(2, 2), rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(kn.norm(dim=-1), torch.ones(2, 2), rtol=1e-5, atol=1e-5)
+    o1, s1 = gdn.gdn_decode_fused_step(qr, kr, v, a, b, a_log, dt_bias, state.clone())
+    o2, s2 = gdn.gdn_decode_fused_step(7.0 * qr, 0.25 * kr, v, a, b, a_log, dt_bias, state.clone())
+    torch.testing.assert_close(o1, o2, rtol=1e-4, atol=1e-6)      # up to the 1e-6 under the root
+    torch.testing.assert_close(s1, s2, rtol=1e-4, atol=1e-6)
+
+
+def test_prestep_limits():
+    gen = torch.Generator().manual_seed(23)
+    qr, kr, v, a, b, a_log, dt_bias, state = gdn.gdn_make_raw_inputs(2, 4, 4, 16, 8, generator=gen)
+    _, _, g, _ = gdn.gdn_prestep(qr, kr, a, b, torch.full_like(a_log, -60.0), dt_bias)
+    assert torch.equal(g, torch.ones_like(g))                    # no decay
+    _, _, _, beta = gdn.gdn_prestep(qr, kr, a, torch.full_like(b, -100.0), a_log, dt_bias)
+    assert torch.equal(beta, torch.zeros_like(beta))             # nothing is written
+    o, s = gdn.gdn_decode_fused_step(qr, kr, v, a, torch.full_like(b, -100.0), torch.full_like(a_log, -60.0),
+                                     dt_bias, state.clone())
+    assert torch.equal(s, state)
+
+
+def test_fused_step_is_prestep_then_step():
+    gen = torch.Generator().manual_seed(24)
+    qr, kr, v, a, b, a_log, dt_bias, state = gdn.gdn_make_raw_inputs(2, 6, 3, 32, 16, generator=gen)
+    qn, kn, g, beta = gdn.gdn_prestep(qr, kr, a, b, a_log, dt_bias)
+    want_o, want_s = gdn.gdn_decode_loops_f64(qn, kn, v, g, beta, state)
+    o, s = gdn.gdn_decode_fused_step(qr, kr, v, a, b, a_log, dt_bias, state.clone())
+    np.testing.assert_allclose(o.numpy(), want_o, rtol=1e-4, atol=1e-6)
+    np.testing.assert_allclose(s.numpy(), want_s, rtol=1e-4, atol=1e-6)
+
+
+def test_fused_golden_fixture_from_third_party_layer_functions():
+    z = np.load(FUSED_GOLDEN)
+    ins = [torch.from_numpy(z[n]) for n in ('q', 'k', 'v', 'a', 'b', 'a_log', 'dt_bias', 'state')]
+    o, s = gdn.gdn_decode_fused_step(*ins[:7], ins[7].clone())
+    np.testing.assert_allclose(o.numpy(), z['o'], rtol=5e-5, atol=2e-7)
+    np.testing.assert_allclose(s.numpy(), z['new_state'], rtol=5e-5, atol=2e-7)
