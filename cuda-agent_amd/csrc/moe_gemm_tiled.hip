@@ -3,8 +3,8 @@
 // A workgroup of 8 wavefronts computes a 256 (weight rows) x 256 (pairs) tile of one expert:
 // per 128-block of K it brings 32 KB of weights, 32 KB of activations and the 256 activation
 // scales of the block into LDS with global->LDS loads in which 8 lanes fetch one full 128-byte
-// line of a row (two stages: the next block loads while the current one is multiplied), and
-// each wavefront multiplies a 64-row x 128-pair slice on v_mfma_f32_32x32x64_f8f6f4:
+// line of a row (two stages; weights are requested two blocks ahead and activations one, see
+// the comment at `block` in the kernel), and each wavefront multiplies a 64-row x 128-pair slice on v_mfma_f32_32x32x64_f8f6f4:
 //
 //   weights are the A operand (rows -> M), activations the B operand (pairs -> N), so that in the
 //   result layout a lane holds 16 weight rows of ONE pair and the block's scale product

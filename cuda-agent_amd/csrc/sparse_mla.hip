@@ -26,6 +26,11 @@
 //     registers.
 // Each split writes a normalised partial output and its log2-sum-exp; a merge kernel combines
 // the splits and converts to bf16.
+//
+// Two split kernels share this data path. sparse_mla_split_kernel<NW> is the form described
+// above (one wavefront per 32 heads; used for 32 and 64 heads and for caches of 4 GB and more
+// per request). sparse_mla_split8_kernel, further down, is the default for multiples of 128
+// heads: two wavefronts per 32 heads that split Q by d and the accumulator by dv.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
