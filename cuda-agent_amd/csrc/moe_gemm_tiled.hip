@@ -505,7 +505,8 @@ extern "C" void moe_gate_up_tiled_launcher(void* h_q, float* h_s, float* hs_t, c
                                            int n_experts, int top_k, int scale_stride,
                                            hipStream_t stream) {
     if (tokens <= 0) return;
-    if (hidden % GROUP != 0 || inter % GROUP != 0 || hidden <= 0 || inter <= 0) {
+    if (hidden % GROUP != 0 || inter % GROUP != 0 || hidden <= 0 || inter <= 0 ||
+        (unsigned long long)tokens * hidden >= (1ull << 32)) {  // 32-bit activation offsets
         caa::set_status(CAA_UNSUPPORTED_SHAPE);
         return;
     }
@@ -522,7 +523,8 @@ extern "C" void moe_down_tiled_launcher(float* y, const void* h_q, const float* 
                                         const int* tile_start, int tokens, int hidden, int inter,
                                         int n_experts, int top_k, int scale_stride, hipStream_t stream) {
     if (tokens <= 0) return;
-    if (hidden % TILE_ROWS != 0 || inter % GROUP != 0 || hidden <= 0 || inter <= 0) {
+    if (hidden % TILE_ROWS != 0 || inter % GROUP != 0 || hidden <= 0 || inter <= 0 ||
+        (unsigned long long)tokens * top_k * inter >= (1ull << 32)) {  // 32-bit activation offsets
         caa::set_status(CAA_UNSUPPORTED_SHAPE);
         return;
     }

@@ -158,8 +158,11 @@ extern "C" void moe_fp8_launcher(void* out, const void* x, const float* logits, 
                             logits, tokens, n_experts, top_k, 0, stream);
     moe_quant_bf16_launcher(w.x_q, w.x_s, x, tokens, hidden, 0, stream);
     // Many pairs per expert: LDS-tiled GEMMs (256 x 256 tiles). Few: the weight-streaming form.
+    // (the tiled kernels address activations with 32-bit byte offsets)
+    const bool fits32 = (unsigned long long)tokens * hidden < (1ull << 32) &&
+                        (unsigned long long)tokens * top_k * inter < (1ull << 32);
     const bool tiled = config == 16 || (config == 0 && (long)tokens * top_k > 32L * n_experts &&
-                                        hidden % 256 == 0);
+                                        hidden % 256 == 0 && fits32);
     if (tiled) {
         moe_tiled_prepare_launcher(w.tile_start, w.xs_t, w.x_s, w.sorted_pairs, w.expert_offsets, tokens,
                                    hidden, n_experts, top_k, w.scale_stride, stream);
