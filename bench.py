@@ -150,7 +150,7 @@ def bench_gdn_fused(torch, capi, dev, steps, warmup, cpu_baseline):
     return res
 
 
-def bench_mla(torch, capi, dev, steps, warmup, cpu_baseline):
+def bench_mla(torch, capi, dev, steps, warmup, cpu_baseline, paged=False):
     from oracle import mla
     B, H, N, topk = 64, 128, 32768, 2048
     gen = torch.Generator(device=dev).manual_seed(20253)
@@ -161,17 +161,27 @@ def bench_mla(torch, capi, dev, steps, warmup, cpu_baseline):
             for _ in range(4)]
     out = torch.empty(B, H, 512, device=dev, dtype=torch.bfloat16)
     ws = torch.empty(capi.sparse_mla_workspace_bytes(B, H, topk), dtype=torch.uint8, device=dev)
-    sec = timed_launches(torch, lambda i: capi.sparse_mla_decode_launch(out, q, kv, idxs[i % 4], ws), steps, warmup)
+    if paged:
+        # the same bytes seen as one pool of 64-row pages; every request's block table maps its 512
+        # logical pages to random pages of the pool
+        page = 64
+        pool = kv.view(B * N // page, page, 576)
+        table = torch.randperm(B * N // page, device=dev, generator=gen).int().view(B, N // page)
+        launch = lambda i: capi.sparse_mla_decode_paged_launch(out, q, pool, table, idxs[i % 4], ws)
+    else:
+        launch = lambda i: capi.sparse_mla_decode_launch(out, q, kv, idxs[i % 4], ws)
+    sec = timed_launches(torch, launch, steps, warmup)
     work = B * topk * 576 * 2
     flops = 2 * B * H * topk * (576 + 512)
     res = dict(
         workload="configs[3]: sparse-MLA decode B=64, 128 heads, 576-dim latent rows, top-k 2048 of 32768, "
-                 "bf16, seed 20253 (split kernel + merge per step)",
+                 "bf16, seed 20253 (split kernel + merge per step)" +
+                 ("; cache held as one pool of 64-row pages behind a block table" if paged else ""),
         value=work / sec / 1e9, unit="GB/s", ms_per_step=sec * 1e3, dtype="bf16", kernel="sparse_mla_split8_kernel",
         roofline=dict(bound="hbm", achieved=work / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
-                      frac=work / sec / 1e9 / HBM_PEAK_GBS, traffic=MEASURED_TRAFFIC['mla']),
+                      frac=work / sec / 1e9 / HBM_PEAK_GBS, traffic=None if paged else MEASURED_TRAFFIC['mla']),
         algorithmic_bytes=work, tflops=flops / sec / 1e12)
-    if cpu_baseline:
+    if cpu_baseline and not paged:
         cores = len(os.sched_getaffinity(0))
         torch.set_num_threads(cores)
         nb = 8
@@ -267,7 +277,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=20)
     ap.add_argument('--warmup', type=int, default=5)
-    ap.add_argument('--workloads', default='gdn,gdn_fused,moe_decode,mla,moe_prefill')
+    ap.add_argument('--workloads', default='gdn,gdn_fused,moe_decode,mla,mla_paged,moe_prefill')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run 3 plain device copies of 536 870 912 bytes (a kernel of known traffic, '
@@ -302,6 +312,8 @@ def main():
             results[name] = bench_gdn_fused(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'mla':
             results[name] = bench_mla(torch, capi, dev, args.steps, args.warmup, cpu)
+        elif name == 'mla_paged':
+            results[name] = bench_mla(torch, capi, dev, args.steps, args.warmup, cpu, paged=True)
         elif name == 'moe_decode':
             results[name] = bench_moe(torch, capi, dev, args.steps, args.warmup, cpu, prefill=False)
         elif name == 'moe_prefill':

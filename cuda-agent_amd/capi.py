@@ -24,6 +24,9 @@ SIGNATURES = {
                                          c_int, c_int, c_int, _P]),
     'sparse_mla_decode_launcher': (None, [_P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int,
                                           c_int, c_int, c_float, c_int, c_int, _P]),
+    'sparse_mla_decode_paged_launcher': (None, [_P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int,
+                                                c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
+                                                _P]),
     'sparse_mla_decode_num_splits': (c_int, [c_int, c_int, c_int, c_int]),
     'sparse_mla_decode_workspace_bytes': (c_size_t, [c_int, c_int, c_int, c_int]),
     'moe_route_launcher': (None, [_P, _P, _P, c_int, c_int, c_int, c_int, _P]),
@@ -171,6 +174,37 @@ def sparse_mla_decode_launch(out, q, kv, idx, workspace, sm_scale=192 ** -0.5, c
                                          0 if out.dtype == torch.bfloat16 else 1, config,
                                          _stream(stream))
     check_status('sparse_mla_decode_launcher')
+    return out
+
+
+def sparse_mla_decode_paged_launch(out, q, kv_pool, block_table, idx, workspace, sm_scale=192 ** -0.5,
+                                   config=0, stream=None):
+    """As ``sparse_mla_decode_launch`` over a paged cache: kv_pool [n_pages, page_size, 576] bf16,
+    block_table [B, max_pages] int32 or None (idx then holds pool rows), idx [B, topk] int32."""
+    import torch
+    _device_contiguous(out=out, q=q, kv_pool=kv_pool, idx=idx, workspace=workspace)
+    B, H, d_qk = q.shape
+    n_pages, page_size = kv_pool.shape[0], kv_pool.shape[1]
+    topk = idx.shape[1]
+    d_v = out.shape[2]
+    _require(q.dtype == kv_pool.dtype == torch.bfloat16, 'sparse_mla: q, kv_pool must be bf16')
+    _require(out.dtype in (torch.bfloat16, torch.float32), 'sparse_mla: out must be bf16 or fp32')
+    _require(idx.dtype == torch.int32, 'sparse_mla: idx must be int32')
+    _require(tuple(kv_pool.shape) == (n_pages, page_size, d_qk) and tuple(idx.shape) == (B, topk),
+             'sparse_mla: kv_pool/idx shape')
+    _require(tuple(out.shape) == (B, H, d_v), 'sparse_mla: out shape')
+    max_pages = 0
+    if block_table is not None:
+        _device_contiguous(block_table=block_table)
+        _require(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.shape[0] == B,
+                 'sparse_mla: block_table must be int32 [B, max_pages]')
+        max_pages = block_table.shape[1]
+    library().sparse_mla_decode_paged_launcher(
+        _ptr(out), _ptr(q), _ptr(kv_pool), _ptr(block_table) if block_table is not None else None,
+        _ptr(idx), _ptr(workspace), workspace.numel() * workspace.element_size(), B, H, n_pages,
+        page_size, max_pages, topk, d_qk, d_v, float(sm_scale),
+        0 if out.dtype == torch.bfloat16 else 1, config, _stream(stream))
+    check_status('sparse_mla_decode_paged_launcher')
     return out
 
 

@@ -313,12 +313,38 @@ __device__ __forceinline__ void wait_all_memory() {
     __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (0 << 8));
 }
 
+// Where the rows of a request live. Without a block table a request's rows are
+// kv + b * batch_rows * 1152 + key * 1152 (batch_rows == 0: one pool shared by all requests,
+// keys are pool rows). With a block table keys are logical positions of the request and
+// logical page p = key >> page_shift lives at physical page block_table[b * table_stride + p].
+struct KvAddressing {
+    const int* block_table;
+    int table_stride;
+    int page_shift;
+    int batch_rows;
+};
+
+// selected key -> row of the cache block, or -1 for padding (negative keys, keys beyond the
+// block table, unmapped pages, rows beyond the cache)
+__device__ __forceinline__ int resolve_key(int key, int b, const KvAddressing& kva, int n_kv_rows) {
+    if (kva.block_table != nullptr) {
+        const int page_no = key >> kva.page_shift;
+        if (key < 0 || page_no >= kva.table_stride) return -1;
+        const int page = kva.block_table[(size_t)b * kva.table_stride + page_no];
+        if (page < 0) return -1;
+        const long long row =
+            ((long long)page << kva.page_shift) + (key & ((1 << kva.page_shift) - 1));
+        return row < n_kv_rows ? (int)row : -1;
+    }
+    return key >= 0 && key < n_kv_rows ? key : -1;
+}
+
 // grid: x = split, y = request, z = head group of 32*NW heads
 template <int NW>
 __global__ __launch_bounds__(64 * NW) void sparse_mla_split_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ kv, const int* __restrict__ idx,
     float* __restrict__ o_part, float* __restrict__ lse_part, int n_heads, int n_kv_rows, int topk,
-    int rows_per_split, float scale_log2) {
+    int rows_per_split, float scale_log2, KvAddressing kva) {
     constexpr int PER_WAVE = TileLoader<NW>::PER_WAVE;
     // Three separately named tile buffers: the compiler then knows which in-flight
     // global->LDS loads an LDS read can depend on and does not drain all of them.
@@ -345,22 +371,16 @@ __global__ __launch_bounds__(64 * NW) void sparse_mla_split_kernel(
     if (tid == 0) s_first_masked_tile = n_tiles;
     __syncthreads();
     for (int i = tid; i < n_tiles * TILE_ROWS; i += 64 * NW) {
-        int key = -1;
-        if (i < n_rows) {
-            key = idx[(size_t)b * topk + row_begin + i];
-            if (key >= n_kv_rows) key = -1;  // out-of-range selections are treated as padding
-        }
-        if (key < 0) {
-            key = -1;
-            atomicMin(&s_first_masked_tile, i / TILE_ROWS);
-        }
+        int key = -1;  // out-of-range selections are treated as padding
+        if (i < n_rows) key = resolve_key(idx[(size_t)b * topk + row_begin + i], b, kva, n_kv_rows);
+        if (key < 0) atomicMin(&s_first_masked_tile, i / TILE_ROWS);
         s_idx[i] = key;
     }
     __syncthreads();
     const int first_masked_tile = s_first_masked_tile;
 
     const TileLoader<NW> loader{
-        reinterpret_cast<const char*>(kv) + (size_t)b * n_kv_rows * ROW_BYTES, wave, lane};
+        reinterpret_cast<const char*>(kv) + (size_t)b * kva.batch_rows * ROW_BYTES, wave, lane};
 
     // prologue: tiles 0 and 1 in flight
     if (n_tiles > 0) loader.issue_all(tile0, s_idx, 0 >= first_masked_tile);
@@ -542,7 +562,7 @@ __device__ __forceinline__ void gather_issue(uint4* tile, const char* kv_b, uint
 __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ kv, const int* __restrict__ idx,
     float* __restrict__ o_part, float* __restrict__ lse_part, int n_heads, int n_kv_rows, int topk,
-    int rows_per_split, float scale_log2) {
+    int rows_per_split, float scale_log2, KvAddressing kva) {
     typedef const __attribute__((address_space(3))) uintx4* lds_x4;
     typedef shortx4 __attribute__((address_space(3)))* lds_s4;
     __shared__ uint4 tiles[3 * TILE_CHUNKS];  // ring of three resident tiles
@@ -579,6 +599,11 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
         const int i = tid + 512 * j;
         raw_key[j] = i < n_rows ? idx[(size_t)b * topk + row_begin + i] : -1;
     }
+    if (kva.block_table != nullptr) {
+#pragma unroll
+        for (int j = 0; j < MAX_SPLIT_ROWS / 512; ++j)
+            raw_key[j] = resolve_key(raw_key[j], b, kva, n_kv_rows);
+    }
     if (tid == 0) s_first_masked_tile = n_tiles;
     for (int c = tid; c < GATHER_TAB; c += 512) {
         const int row = c / ROW_CHUNKS;  // 0..7; the tile row is 8*quarter + row: for odd quarters the
@@ -601,7 +626,7 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
     }
     __syncthreads();
     const int first_masked_tile = s_first_masked_tile;
-    const char* kv_b = reinterpret_cast<const char*>(kv) + (size_t)b * n_kv_rows * ROW_BYTES;
+    const char* kv_b = reinterpret_cast<const char*>(kv) + (size_t)b * kva.batch_rows * ROW_BYTES;
     PHASE_MARK(7);  // index staging
 
     // The first two tiles are on their way before Q is fetched: tile 0 by the lead group, tile 1
@@ -901,21 +926,14 @@ extern "C" size_t sparse_mla_decode_workspace_bytes(int batch, int n_heads, int 
     return (size_t)batch * splits * n_heads * (D_V + 1) * sizeof(float);
 }
 
-// out  [batch, n_heads, 512], written; bf16 if out_dtype == 0 (the operator's output type),
-//      fp32 if out_dtype == 1 (the same values before the final rounding, for measuring
-//      arithmetic error apart from output rounding)
-// q    [batch, n_heads, 576] bf16
-// kv   [batch, n_kv_rows, 576] bf16 (latent cache: 512 latent + 64 rope dims per row)
-// idx  [batch, topk] int32 row numbers into the request's cache; values < 0 or >= n_kv_rows
-//      are padding and take no part in the softmax
-// workspace: sparse_mla_decode_workspace_bytes(...) bytes of device scratch, 16-byte aligned
-// config: 0 picks the number of key splits so that one workgroup per CU is resident;
-//         n > 0 forces n splits.
-extern "C" void sparse_mla_decode_launcher(void* out, const void* q, const void* kv, const int* idx,
-                                           void* workspace, size_t workspace_bytes, int batch,
-                                           int n_heads, int n_kv_rows, int topk, int d_qk, int d_v,
-                                           float sm_scale, int out_dtype, int config,
-                                           hipStream_t stream) {
+namespace {
+
+// shared by the two launchers: n_kv_rows is the number of rows of the block a request's keys
+// resolve into (the request's own cache, or the whole pool)
+void launch_sparse_mla(void* out, const void* q, const void* kv, const int* idx, void* workspace,
+                       size_t workspace_bytes, int batch, int n_heads, int n_kv_rows, int topk,
+                       int d_qk, int d_v, float sm_scale, int out_dtype, int config,
+                       const KvAddressing& kva, hipStream_t stream) {
     if (batch <= 0 || n_heads <= 0 || topk <= 0) return;
     const bool heads_ok = n_heads == 32 || n_heads == 64 || (n_heads % 128 == 0);
     if (d_qk != D_QK || d_v != D_V || !heads_ok || n_kv_rows <= 0 || batch > 65535 ||
@@ -953,18 +971,19 @@ extern "C" void sparse_mla_decode_launcher(void* out, const void* q, const void*
     if (n_heads == 32) {
         sparse_mla_split_kernel<1><<<grid, 64, 0, stream>>>(qb, kvb, idx, o_part, lse_part, n_heads,
                                                             n_kv_rows, topk, rows_per_split,
-                                                            scale_log2);
+                                                            scale_log2, kva);
     } else if (n_heads == 64) {
         sparse_mla_split_kernel<2><<<grid, 128, 0, stream>>>(qb, kvb, idx, o_part, lse_part, n_heads,
                                                              n_kv_rows, topk, rows_per_split,
-                                                             scale_log2);
+                                                             scale_log2, kva);
     } else if (four_wave_kernel) {
         sparse_mla_split_kernel<4><<<grid, 256, 0, stream>>>(qb, kvb, idx, o_part, lse_part, n_heads,
                                                              n_kv_rows, topk, rows_per_split,
-                                                             scale_log2);
+                                                             scale_log2, kva);
     } else {
         sparse_mla_split8_kernel<<<grid, 512, 0, stream>>>(qb, kvb, idx, o_part, lse_part, n_heads,
-                                                           n_kv_rows, topk, rows_per_split, scale_log2);
+                                                           n_kv_rows, topk, rows_per_split,
+                                                           scale_log2, kva);
     }
     if (out_dtype == 0) {
         sparse_mla_merge_kernel<__bf16><<<dim3(n_heads, batch), 128, 0, stream>>>(
@@ -973,4 +992,58 @@ extern "C" void sparse_mla_decode_launcher(void* out, const void* q, const void*
         sparse_mla_merge_kernel<float><<<dim3(n_heads, batch), 128, 0, stream>>>(
             o_part, lse_part, static_cast<float*>(out), n_heads, splits);
     }
+}
+
+}  // namespace
+
+// out  [batch, n_heads, 512], written; bf16 if out_dtype == 0 (the operator's output type),
+//      fp32 if out_dtype == 1 (the same values before the final rounding, for measuring
+//      arithmetic error apart from output rounding)
+// q    [batch, n_heads, 576] bf16
+// kv   [batch, n_kv_rows, 576] bf16 (latent cache: 512 latent + 64 rope dims per row)
+// idx  [batch, topk] int32 row numbers into the request's cache; values < 0 or >= n_kv_rows
+//      are padding and take no part in the softmax
+// workspace: sparse_mla_decode_workspace_bytes(...) bytes of device scratch, 16-byte aligned
+// config: 0 picks the number of key splits so that one workgroup per CU is resident;
+//         n > 0 forces n splits.
+extern "C" void sparse_mla_decode_launcher(void* out, const void* q, const void* kv, const int* idx,
+                                           void* workspace, size_t workspace_bytes, int batch,
+                                           int n_heads, int n_kv_rows, int topk, int d_qk, int d_v,
+                                           float sm_scale, int out_dtype, int config,
+                                           hipStream_t stream) {
+    const KvAddressing kva{nullptr, 0, 0, n_kv_rows};
+    launch_sparse_mla(out, q, kv, idx, workspace, workspace_bytes, batch, n_heads, n_kv_rows, topk,
+                      d_qk, d_v, sm_scale, out_dtype, config, kva, stream);
+}
+
+// The same attention over a paged latent cache: one pool of pages shared by all requests.
+// kv_pool     [n_pages, page_size, 576] bf16, page_size a power of two
+// block_table [batch, max_pages_per_request] int32: physical page of each logical page of a
+//             request, negative where no page is mapped; or null
+// idx         [batch, topk] int32. With a block table: logical positions of the request
+//             (position p is row p % page_size of page block_table[b][p / page_size]). Without:
+//             rows of the pool, page * page_size + row, as an indexer that already works on
+//             physical rows hands them over. Negative entries, positions beyond the block
+//             table, unmapped pages and rows beyond the pool are padding.
+// Everything else as sparse_mla_decode_launcher; the workspace size is the same function of
+// (batch, n_heads, topk, config).
+extern "C" void sparse_mla_decode_paged_launcher(void* out, const void* q, const void* kv_pool,
+                                                 const int* block_table, const int* idx,
+                                                 void* workspace, size_t workspace_bytes, int batch,
+                                                 int n_heads, int n_pages, int page_size,
+                                                 int max_pages_per_request, int topk, int d_qk,
+                                                 int d_v, float sm_scale, int out_dtype, int config,
+                                                 hipStream_t stream) {
+    if (batch <= 0 || n_heads <= 0 || topk <= 0) return;
+    if (n_pages <= 0 || page_size <= 0 || (page_size & (page_size - 1)) != 0 ||
+        (long long)n_pages * page_size > 0x7fffffffll ||
+        (block_table != nullptr && max_pages_per_request <= 0)) {
+        caa::set_status(CAA_UNSUPPORTED_SHAPE);
+        return;
+    }
+    int page_shift = 0;
+    while ((1 << page_shift) < page_size) ++page_shift;
+    const KvAddressing kva{block_table, max_pages_per_request, page_shift, 0};
+    launch_sparse_mla(out, q, kv_pool, idx, workspace, workspace_bytes, batch, n_heads,
+                      n_pages * page_size, topk, d_qk, d_v, sm_scale, out_dtype, config, kva, stream);
 }

@@ -104,6 +104,29 @@ void sparse_mla_decode_launcher(void* out, const void* q, const void* kv, const 
                                 int n_kv_rows, int topk, int d_qk, int d_v, float sm_scale,
                                 int out_dtype, int config, hipStream_t stream);
 
+/* The same attention over a paged latent cache, the layout a serving engine keeps (one pool of
+ * fixed-size pages shared by all requests and a block table per request). Same launcher pattern
+ * (agent_workdir/kernels/axpby.cu:12-20); the operator is the caller-side neighbour of the one
+ * above, not a separate workload of the benchmark definition.
+ *   kv_pool     [n_pages, page_size, 576] bf16; page_size a power of two,
+ *               n_pages * page_size < 2^31
+ *   block_table [batch, max_pages_per_request] int32, physical page of each logical page of a
+ *               request, negative = not mapped; or NULL
+ *   idx         [batch, topk] int32. With a block table: logical positions of the request;
+ *               position p is row p % page_size of page block_table[b][p / page_size].
+ *               With block_table == NULL: rows of the pool (page * page_size + row).
+ *               Negative entries, positions beyond the block table, unmapped pages and rows
+ *               beyond the pool are padding and are skipped.
+ * Everything else (out, q, workspace and its size, sm_scale, out_dtype, config, supported
+ * shapes) as for sparse_mla_decode_launcher. A pool of 4 GB or more is served by the kernel with
+ * one wavefront per 32 heads. */
+void sparse_mla_decode_paged_launcher(void* out, const void* q, const void* kv_pool,
+                                      const int* block_table, const int* idx, void* workspace,
+                                      size_t workspace_bytes, int batch, int n_heads, int n_pages,
+                                      int page_size, int max_pages_per_request, int topk, int d_qk,
+                                      int d_v, float sm_scale, int out_dtype, int config,
+                                      hipStream_t stream);
+
 /* Number of key splits the launcher will use for these sizes and this config. */
 int sparse_mla_decode_num_splits(int batch, int n_heads, int topk, int config);
 

@@ -17,6 +17,13 @@ Pinned by (tests/test_oracle_mla.py):
     shared KV head;
   * invariants: permutation of idx, all-equal V rows, shift invariance, split-and-merge by
     log-sum-exp.
+
+Paged cache (the serving-side layout next to the operator; no counterpart in the reference
+repository either): ``resolve_paged_indices`` maps logical positions through a block table,
+position p of request b -> row ``p % page_size`` of page ``block_table[b, p // page_size]`` of
+one pool shared by all requests. Pinned by scalar loops over divmod on small cases and by the
+identity "scatter a contiguous cache's pages into a pool under a random page permutation ->
+the paged result equals the contiguous result exactly".
 """
 
 import math
@@ -71,6 +78,48 @@ def mla_make_inputs(batch, n_heads, n_kv_rows, topk, generator=None, device='cpu
     idx = torch.stack([torch.randperm(n_kv_rows, generator=gen, device=device)[:topk]
                        for _ in range(batch)]).int()
     return [q, kv, idx]
+
+
+def resolve_paged_indices(idx, block_table, page_size, n_pool_rows):
+    """Logical positions idx [B,topk] -> rows of the pool (int64), -1 for padding: negative
+    positions, positions beyond the block table, unmapped (negative) pages, rows beyond the
+    pool. With ``block_table=None`` idx already holds pool rows and only the range check
+    applies."""
+    idx = idx.long()
+    if block_table is None:
+        rows = idx
+    else:
+        max_pages = block_table.shape[1]
+        page_no = torch.div(idx, page_size, rounding_mode='floor')
+        inside = (idx >= 0) & (page_no < max_pages)
+        page = torch.gather(block_table.long(), 1, page_no.clamp(0, max_pages - 1))
+        rows = page * page_size + torch.remainder(idx, page_size)
+        rows = torch.where(inside & (page >= 0), rows, torch.full_like(rows, -1))
+    return torch.where((rows >= 0) & (rows < n_pool_rows), rows, torch.full_like(rows, -1))
+
+
+def sparse_mla_decode_paged(q, kv_pool, block_table, idx, sm_scale=SM_SCALE, out_dtype=torch.bfloat16):
+    """q [B,H,576], kv_pool [n_pages,page_size,576], block_table [B,max_pages] or None,
+    idx [B,topk] -> out [B,H,512]: the attention of ``sparse_mla_decode`` over the rows the
+    block table resolves to."""
+    n_pages, page_size, d = kv_pool.shape
+    rows = resolve_paged_indices(idx, block_table, page_size, n_pages * page_size)
+    pool = kv_pool.reshape(1, n_pages * page_size, d).expand(q.shape[0], -1, -1)
+    return sparse_mla_decode(q, pool, rows, sm_scale, out_dtype)
+
+
+def mla_scatter_into_pool(kv, page_size, n_spare_pages=3, generator=None):
+    """A contiguous cache kv [B,N,576] (N a multiple of page_size) cut into pages and placed in a
+    pool at randomly permuted page numbers, with a few unused pages of noise in between.
+    Returns (kv_pool [n_pages,page_size,576], block_table [B, N/page_size] int32)."""
+    B, N, d = kv.shape
+    assert N % page_size == 0
+    per_req = N // page_size
+    n_pages = B * per_req + n_spare_pages
+    order = torch.randperm(n_pages, generator=generator)[:B * per_req]
+    pool = torch.randn(n_pages, page_size, d, generator=generator).to(kv.dtype)
+    pool[order] = kv.reshape(B * per_req, page_size, d).cpu()
+    return pool, order.reshape(B, per_req).int()
 
 
 def rel_rms_error(actual, expected):

@@ -80,3 +80,60 @@ def test_output_dtype_and_shape():
     assert idx.dtype == torch.int32
     for b in range(2):
         assert len(set(idx[b].tolist())) == idx.shape[1]
+
+
+# ---- paged cache ------------------------------------------------------------------------------
+
+def _resolve_by_loops(idx, block_table, page_size, n_pool_rows):
+    out = []
+    for b, row in enumerate(idx.tolist()):
+        res = []
+        for p in row:
+            r = -1
+            if block_table is None:
+                r = p
+            elif p >= 0:
+                page_no, offset = divmod(p, page_size)
+                if page_no < block_table.shape[1] and int(block_table[b, page_no]) >= 0:
+                    r = int(block_table[b, page_no]) * page_size + offset
+            res.append(r if 0 <= r < n_pool_rows else -1)
+        out.append(res)
+    return torch.tensor(out)
+
+
+def test_paged_resolution_matches_divmod_loops():
+    gen = torch.Generator().manual_seed(5)
+    page_size, n_pages, B, max_pages = 4, 9, 3, 5
+    table = torch.randint(-1, n_pages + 2, (B, max_pages), generator=gen).int()   # unmapped and out-of-pool pages
+    idx = torch.randint(-3, max_pages * page_size + 6, (B, 40), generator=gen).int()
+    got = mla.resolve_paged_indices(idx, table, page_size, n_pages * page_size)
+    assert torch.equal(got, _resolve_by_loops(idx, table, page_size, n_pages * page_size))
+    assert (got == -1).any() and (got >= 0).any()
+    rows = torch.randint(-2, n_pages * page_size + 3, (B, 40), generator=gen).int()
+    got = mla.resolve_paged_indices(rows, None, page_size, n_pages * page_size)
+    assert torch.equal(got, _resolve_by_loops(rows, None, page_size, n_pages * page_size))
+
+
+def test_paged_equals_contiguous_when_the_pool_holds_the_same_pages():
+    gen = torch.Generator().manual_seed(6)
+    q, kv, idx = mla.mla_make_inputs(3, 4, 48, 20, generator=gen)
+    idx[1, 3] = -1
+    idx[2, 7] = 48
+    want = mla.sparse_mla_decode(q, kv, idx, out_dtype=torch.float32)
+    pool, table = mla.mla_scatter_into_pool(kv, 8, generator=gen)
+    got = mla.sparse_mla_decode_paged(q, pool, table, idx, out_dtype=torch.float32)
+    assert torch.equal(got, want)
+    # the same selection handed over as pool rows, without a block table
+    rows = mla.resolve_paged_indices(idx, table, 8, pool.shape[0] * 8).int()
+    assert torch.equal(mla.sparse_mla_decode_paged(q, pool, None, rows, out_dtype=torch.float32), want)
+
+
+def test_unmapped_pages_drop_their_positions():
+    gen = torch.Generator().manual_seed(7)
+    q, kv, idx = mla.mla_make_inputs(2, 4, 32, 16, generator=gen)
+    pool, table = mla.mla_scatter_into_pool(kv, 8, generator=gen)
+    table[0, 1] = -1
+    keep = idx.clone()
+    keep[0][(idx[0] >= 8) & (idx[0] < 16)] = -1
+    want = mla.sparse_mla_decode(q, kv, keep, out_dtype=torch.float32)
+    assert torch.equal(mla.sparse_mla_decode_paged(q, pool, table, idx, out_dtype=torch.float32), want)
