@@ -150,6 +150,40 @@ def bench_gdn_fused(torch, capi, dev, steps, warmup, cpu_baseline):
     return res
 
 
+def bench_conv1d(torch, capi, dev, steps, warmup, cpu_baseline):
+    """The convolution update in front of the configs[1] GDN step: 256 requests, 2*2048 + 4096 channels,
+    4 taps, a 4-column state per channel, bf16."""
+    from oracle import gdn
+    B, key_dim, value_dim, L, K = 256, 2048, 4096, 4, 4
+    C = 2 * key_dim + value_dim
+    gen = torch.Generator().manual_seed(20257)
+    host = gdn.conv_make_inputs(B, key_dim, value_dim, L, K, torch.bfloat16, generator=gen)
+    x, state0, weight, bias = (t.to(dev) for t in host)
+    # 24 state copies (403 MB): one 17 MB state would be served from the cache
+    states = [state0.clone() for _ in range(24)]
+    q = torch.empty(B, key_dim, dtype=torch.bfloat16, device=dev)
+    k = torch.empty_like(q)
+    v = torch.empty(B, value_dim, dtype=torch.bfloat16, device=dev)
+    sec = timed_launches(
+        torch, lambda i: capi.causal_conv1d_update_launch(q, k, v, states[i % 24], x, weight, bias), steps, warmup)
+    work = B * C * (2 * L + 2) * 2 + C * (K + 1) * 2
+    res = dict(
+        workload="single-token causal convolution update in front of configs[1]: B=256, 8192 channels, 4 taps, "
+                 "4-column bf16 state, SiLU, seed 20257",
+        value=work / sec / 1e9, unit="GB/s", ms_per_step=sec * 1e3, dtype="f32",
+        kernel="causal_conv1d_update_kernel",
+        roofline=dict(bound="hbm", achieved=work / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
+                      frac=work / sec / 1e9 / HBM_PEAK_GBS, traffic=None),
+        algorithmic_bytes=work)
+    if cpu_baseline:
+        cores = len(os.sched_getaffinity(0))
+        torch.set_num_threads(cores)
+        csec = cpu_time(lambda: gdn.causal_conv1d_update(*host))
+        res['cpu_baseline'] = dict(value=work / csec / 1e9, unit="GB/s", cores=cores, kind="port",
+                                   sample="the full update (eager PyTorch oracle, state in place)")
+    return res
+
+
 def bench_mla(torch, capi, dev, steps, warmup, cpu_baseline, paged=False):
     from oracle import mla
     B, H, N, topk = 64, 128, 32768, 2048
@@ -277,7 +311,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=20)
     ap.add_argument('--warmup', type=int, default=5)
-    ap.add_argument('--workloads', default='gdn,gdn_fused,moe_decode,mla,mla_paged,moe_prefill')
+    ap.add_argument('--workloads', default='gdn,gdn_fused,conv1d,moe_decode,mla,mla_paged,moe_prefill')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run 3 plain device copies of 536 870 912 bytes (a kernel of known traffic, '
@@ -310,6 +344,8 @@ def main():
             results[name] = bench_gdn(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'gdn_fused':
             results[name] = bench_gdn_fused(torch, capi, dev, args.steps, args.warmup, cpu)
+        elif name == 'conv1d':
+            results[name] = bench_conv1d(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'mla':
             results[name] = bench_mla(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'mla_paged':

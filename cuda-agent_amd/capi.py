@@ -22,6 +22,8 @@ SIGNATURES = {
                                    c_int, c_int, _P]),
     'gdn_decode_fused_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int,
                                          c_int, c_int, c_int, _P]),
+    'causal_conv1d_update_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int,
+                                             c_int, c_int, c_int, _P]),
     'sparse_mla_decode_launcher': (None, [_P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int,
                                           c_int, c_int, c_float, c_int, c_int, _P]),
     'sparse_mla_decode_paged_launcher': (None, [_P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int,
@@ -148,6 +150,41 @@ def gdn_decode_fused_launch(o, state, q, k, v, a, b, a_log, dt_bias, config=0, s
                                         0 if q.dtype == torch.float32 else 1, config, _stream(stream))
     check_status('gdn_decode_fused_launcher')
     return o, state
+
+
+def causal_conv1d_update_launch(q_out, k_out, v_out, conv_state, x, weight, bias=None, activation='silu',
+                                config=0, stream=None):
+    """conv_state [B,C,L] shifted in place by x [B,C]; q_out [B,key_dim], k_out [B,key_dim],
+    v_out [B,C-2*key_dim] <- activation(bias + the K newest values . weight [C,K]).
+    q_out = k_out = None puts every channel into v_out."""
+    import torch
+    tensors = dict(v_out=v_out, conv_state=conv_state, x=x, weight=weight)
+    if q_out is not None:
+        tensors.update(q_out=q_out, k_out=k_out)
+    if bias is not None:
+        tensors['bias'] = bias
+    _device_contiguous(**tensors)
+    B, C, L = conv_state.shape
+    K = weight.shape[1]
+    key_dim = 0 if q_out is None else q_out.shape[1]
+    value_dim = v_out.shape[1]
+    dt = conv_state.dtype
+    _require(dt in (torch.float32, torch.bfloat16) and all(t.dtype == dt for t in tensors.values()),
+             'causal_conv1d_update: all tensors fp32 or all bf16')
+    _require(2 * key_dim + value_dim == C and tuple(x.shape) == (B, C) and tuple(weight.shape) == (C, K)
+             and tuple(v_out.shape) == (B, value_dim), 'causal_conv1d_update: shapes')
+    _require(q_out is None or (tuple(q_out.shape) == tuple(k_out.shape) == (B, key_dim)),
+             'causal_conv1d_update: q_out/k_out shape')
+    _require(bias is None or tuple(bias.shape) == (C,), 'causal_conv1d_update: bias shape')
+    _require(activation in (None, 'silu'), "causal_conv1d_update: activation is None or 'silu'")
+    null = c_void_p(None)
+    library().causal_conv1d_update_launcher(
+        _ptr(q_out) if q_out is not None else null, _ptr(k_out) if q_out is not None else null, _ptr(v_out),
+        _ptr(conv_state), _ptr(x), _ptr(weight), _ptr(bias) if bias is not None else null, B, key_dim,
+        value_dim, L, K, 1 if activation == 'silu' else 0, 0 if dt == torch.float32 else 1, config,
+        _stream(stream))
+    check_status('causal_conv1d_update_launcher')
+    return q_out, k_out, v_out
 
 
 def sparse_mla_workspace_bytes(batch, n_heads, topk, config=0):

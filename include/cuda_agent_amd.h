@@ -80,6 +80,25 @@ void gdn_decode_fused_launcher(float* o, float* state, const void* q, const void
                                const float* dt_bias, int batch, int n_v_heads, int n_qk_heads,
                                int dk, int dv, int qkv_dtype, int config, hipStream_t stream);
 
+/* Short causal depthwise convolution, single-token update: the step before the GDN decode step
+ * in a Qwen3-Next-style layer (launcher pattern agent_workdir/kernels/axpby.cu:12-20; not one of
+ * the benchmark's workloads, the caller-side neighbour of gdn_decode_fused_launcher). Per request
+ * b and channel c of the concatenated q|k|v projection:
+ *   seq = [conv_state[b,c,0..L-1], x[b,c]];  conv_state[b,c,:] <- seq[1..L]   (in place)
+ *   y   = bias[c] + sum_{j<K} weight[c,j] * seq[L+1-K+j];  out = y*sigmoid(y) or y
+ *   channels [0,key_dim) -> q_out [batch,key_dim], [key_dim,2*key_dim) -> k_out [batch,key_dim],
+ *   the rest -> v_out [batch,value_dim]
+ *   conv_state [batch, 2*key_dim+value_dim, L], x [batch, 2*key_dim+value_dim],
+ *   weight [2*key_dim+value_dim, K], bias [2*key_dim+value_dim] or NULL
+ * dtype: storage type of every array, 0 = fp32, 1 = bf16 (arithmetic is fp32; the state is moved,
+ * so it stays bit-exact). activation: 0 none, 1 SiLU. Supported: K = kernel_size in 2..4,
+ * L = state_len = K-1 or K, key_dim and value_dim multiples of 8 (key_dim 0: one output, q_out
+ * and k_out may be NULL), batch <= 65535, all pointers 16-byte aligned. config: one value (0). */
+void causal_conv1d_update_launcher(void* q_out, void* k_out, void* v_out, void* conv_state,
+                                   const void* x, const void* weight, const void* bias, int batch,
+                                   int key_dim, int value_dim, int state_len, int kernel_size,
+                                   int activation, int dtype, int config, hipStream_t stream);
+
 /* Sparse-MLA decode attention (workload config 3 of the benchmark definition; launcher
  * pattern agent_workdir/kernels/axpby.cu:12-20). Per request every head attends to the rows
  * of that request's latent cache listed in idx:

@@ -24,6 +24,13 @@ invariance of the normalised vectors, ``softplus``/``sigmoid``/``rsqrt`` library
 float64 closed forms, limits (a_log -> -inf gives g = 1), and a second golden fixture from the same
 third-party function called with its in-kernel L2 normalisation switched on and the gate computed by
 library calls (tests/golden/make_gdn_golden.py, ``gdn_fused_golden.npz``).
+
+``causal_conv1d_update`` is the step before that one in the same layer (short depthwise causal
+convolution over the q|k|v projection, single token, state shifted in place). Pinned by: scalar
+loops, the library convolution ``F.conv1d(groups=C)`` over the concatenated sequence, the identity
+"feeding a sequence token by token equals one causal convolution of the whole sequence", and a
+golden fixture from the third-party layer's own single-token update
+(``conv1d_update_golden.npz``, same generator script).
 """
 
 import math
@@ -94,6 +101,35 @@ def gdn_make_raw_inputs(batch, n_v_heads, n_qk_heads, dk=128, dv=128, qkv_dtype=
     dt_bias = 2 * torch.rand(n_v_heads, generator=gen) - 1
     state = 0.02 * torch.randn(batch, n_v_heads, dk, dv, generator=gen)
     return [q.to(qkv_dtype), k.to(qkv_dtype), v.to(qkv_dtype), a, b, a_log, dt_bias, state]
+
+
+def causal_conv1d_update(x, conv_state, weight, bias=None, activation='silu'):
+    """x [B,C], conv_state [B,C,L] (oldest first, shifted in place), weight [C,K], bias [C] or None.
+    Returns out [B,C] in x's dtype: activation(bias + sum_j weight[:,j] * seq[:, :, L+1-K+j]) with
+    seq = [conv_state, x]; fp32 arithmetic, one rounding at the end."""
+    L = conv_state.shape[2]
+    K = weight.shape[1]
+    assert L >= K - 1
+    seq = torch.cat([conv_state, x[:, :, None]], dim=2)
+    conv_state.copy_(seq[:, :, 1:])
+    y = (seq[:, :, L + 1 - K:].float() * weight.float()[None]).sum(dim=2)
+    if bias is not None:
+        y = y + bias.float()[None]
+    if activation == 'silu':
+        y = y * torch.sigmoid(y)
+    return y.to(x.dtype)
+
+
+def conv_make_inputs(batch, key_dim, value_dim, state_len=4, kernel_size=4, dtype=torch.bfloat16,
+                     generator=None, device='cpu'):
+    """x, conv_state ~ N(0,1), weight ~ N(0, 1/K), bias ~ 0.1 N(0,1), all cast to ``dtype``."""
+    C = 2 * key_dim + value_dim
+    gen = generator
+    x = torch.randn(batch, C, generator=gen, device=device).to(dtype)
+    conv_state = torch.randn(batch, C, state_len, generator=gen, device=device).to(dtype)
+    weight = (torch.randn(C, kernel_size, generator=gen, device=device) * kernel_size ** -0.5).to(dtype)
+    bias = (0.1 * torch.randn(C, generator=gen, device=device)).to(dtype)
+    return x, conv_state, weight, bias
 
 
 def gdn_decode_loops_f64(q, k, v, g, beta, state):

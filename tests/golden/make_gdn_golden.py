@@ -1,4 +1,5 @@
-"""Writes tests/golden/gdn_decode_golden.npz from an independent implementation of the gated
+"""Writes tests/golden/gdn_decode_golden.npz (and the two fixtures described further down, for the
+fused pre-step and for the convolution update) from an independent implementation of the gated
 delta rule: the eager ``torch_recurrent_gated_delta_rule`` of the locally installed third-party
 ``transformers`` package (models/qwen3_next/modeling_qwen3_next.py), called with a sequence of
 length 1. That function takes [B, T, H, d] tensors, the decay as a log and ungrouped heads, so
@@ -47,6 +48,25 @@ def main():
     np.savez_compressed(out, q=qr.numpy(), k=kr.numpy(), v=v.numpy(), a=a.numpy(), b=b.numpy(),
                         a_log=a_log.numpy(), dt_bias=dt_bias.numpy(), state=state.numpy(),
                         o=o[:, 0].numpy(), new_state=new_state.numpy())
+    print('wrote', out, out.stat().st_size, 'bytes')
+
+    # the layer's single-token convolution update (fp32; state of K and of K-1 columns, with and
+    # without bias): three consecutive tokens through the third-party function
+    from transformers.models.qwen3_next.modeling_qwen3_next import causal_conv1d_update
+    from oracle.gdn import conv_make_inputs
+    gen = torch.Generator().manual_seed(454545)
+    arrays = {}
+    for tag, L, K, with_bias in (('a', 4, 4, True), ('b', 3, 4, False), ('c', 2, 2, True)):
+        x, conv_state, weight, bias = conv_make_inputs(2, 8, 16, L, K, torch.float32, generator=gen)
+        xs = [x, torch.randn(x.shape, generator=gen), torch.randn(x.shape, generator=gen)]
+        arrays.update({f'{tag}_state0': conv_state.numpy().copy(), f'{tag}_weight': weight.numpy(),
+                       f'{tag}_bias': bias.numpy() if with_bias else np.zeros(0, np.float32)})
+        for t, xt in enumerate(xs):
+            y = causal_conv1d_update(xt[:, :, None], conv_state, weight, bias if with_bias else None, 'silu')
+            arrays.update({f'{tag}_x{t}': xt.numpy(), f'{tag}_out{t}': y[:, :, 0].numpy(),
+                           f'{tag}_state{t + 1}': conv_state.numpy().copy()})
+    out = Path(__file__).with_name('conv1d_update_golden.npz')
+    np.savez_compressed(out, **arrays)
     print('wrote', out, out.stat().st_size, 'bytes')
 
 

@@ -1,12 +1,15 @@
 """Pins the GDN decode oracle: brute force, invariants and a third-party golden fixture."""
+import math
 from pathlib import Path
 
 import numpy as np
+import pytest
 import torch
 
 from oracle import gdn
 
-GOLDEN = Path(__file__).parent / 'golden' / 'gdn_decode_golden.npz'
+GOLDEN_DIR = Path(__file__).parent / 'golden'
+GOLDEN = GOLDEN_DIR / 'gdn_decode_golden.npz'
 
 
 def _tiny(seed=0, B=2, Hv=4, Hqk=2, dk=8, dv=4):
@@ -165,3 +168,76 @@ def test_fused_golden_fixture_from_third_party_layer_functions():
     o, s = gdn.gdn_decode_fused_step(*ins[:7], ins[7].clone())
     np.testing.assert_allclose(o.numpy(), z['o'], rtol=5e-5, atol=2e-7)
     np.testing.assert_allclose(s.numpy(), z['new_state'], rtol=5e-5, atol=2e-7)
+
+
+# ---- single-token causal convolution update ----------------------------------------------------
+
+def _conv_loops(x, state, weight, bias, activation):
+    B, C, L = state.shape
+    K = weight.shape[1]
+    out = np.zeros((B, C))
+    new_state = np.zeros((B, C, L))
+    for b in range(B):
+        for c in range(C):
+            seq = [float(state[b, c, i]) for i in range(L)] + [float(x[b, c])]
+            y = float(bias[c]) if bias is not None else 0.0
+            for j in range(K):
+                y += float(weight[c, j]) * seq[len(seq) - K + j]
+            out[b, c] = y / (1.0 + math.exp(-y)) if activation == 'silu' else y
+            new_state[b, c] = seq[1:]
+    return out, new_state
+
+
+@pytest.mark.parametrize('L,K', [(4, 4), (3, 4), (2, 2), (1, 2), (3, 3)])
+@pytest.mark.parametrize('activation', ['silu', None])
+def test_conv_update_matches_scalar_loops(L, K, activation):
+    gen = torch.Generator().manual_seed(10 * L + K)
+    x, state, weight, bias = gdn.conv_make_inputs(2, 8, 8, L, K, torch.float32, generator=gen)
+    want_out, want_state = _conv_loops(x.numpy(), state.numpy(), weight.numpy(), bias.numpy(), activation)
+    out = gdn.causal_conv1d_update(x, state, weight, bias, activation)
+    np.testing.assert_allclose(out.numpy(), want_out, rtol=1e-5, atol=1e-6)
+    np.testing.assert_array_equal(state.numpy(), want_state.astype(np.float32))
+
+
+def test_conv_update_is_the_library_convolution_of_the_concatenated_sequence():
+    gen = torch.Generator().manual_seed(3)
+    x, state, weight, bias = gdn.conv_make_inputs(3, 8, 16, 4, 4, torch.float32, generator=gen)
+    seq = torch.cat([state, x[:, :, None]], dim=2)
+    want = torch.nn.functional.conv1d(seq, weight[:, None, :], bias, groups=seq.shape[1])[:, :, -1]
+    out = gdn.causal_conv1d_update(x, state, weight, bias, None)
+    torch.testing.assert_close(out, want, rtol=1e-5, atol=1e-6)
+
+
+def test_conv_token_by_token_equals_one_causal_convolution():
+    gen = torch.Generator().manual_seed(4)
+    C, K, T = 16, 4, 9
+    xs = torch.randn(2, C, T, generator=gen)
+    weight = torch.randn(C, K, generator=gen)
+    want = torch.nn.functional.conv1d(torch.nn.functional.pad(xs, (K - 1, 0)), weight[:, None, :], groups=C)
+    for L in (K - 1, K):
+        state = torch.zeros(2, C, L)
+        got = torch.stack([gdn.causal_conv1d_update(xs[:, :, t].contiguous(), state, weight, None, None)
+                           for t in range(T)], dim=2)
+        torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-6)
+        assert torch.equal(state, xs[:, :, T - L:])
+
+
+def test_conv_update_matches_third_party_golden():
+    z = np.load(GOLDEN_DIR / 'conv1d_update_golden.npz')
+    for tag in 'abc':
+        state = torch.from_numpy(z[f'{tag}_state0']).clone()
+        weight = torch.from_numpy(z[f'{tag}_weight'])
+        bias = torch.from_numpy(z[f'{tag}_bias']) if z[f'{tag}_bias'].size else None
+        for t in range(3):
+            out = gdn.causal_conv1d_update(torch.from_numpy(z[f'{tag}_x{t}']), state, weight, bias, 'silu')
+            np.testing.assert_allclose(out.numpy(), z[f'{tag}_out{t}'], rtol=1e-5, atol=1e-6)
+            np.testing.assert_array_equal(state.numpy(), z[f'{tag}_state{t + 1}'])
+
+
+def test_conv_update_rounds_once_for_bf16():
+    gen = torch.Generator().manual_seed(5)
+    x, state, weight, bias = gdn.conv_make_inputs(2, 8, 8, 4, 4, torch.bfloat16, generator=gen)
+    exact = gdn.causal_conv1d_update(x.float(), state.float().clone(), weight.float(), bias.float())
+    out = gdn.causal_conv1d_update(x, state, weight, bias)
+    assert out.dtype == torch.bfloat16 and state.dtype == torch.bfloat16
+    assert torch.equal(out, exact.bfloat16())
