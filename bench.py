@@ -292,6 +292,24 @@ def bench_moe(torch, capi, dev, steps, warmup, cpu_baseline, prefill):
             roofline=dict(bound="hbm", achieved=wbytes / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
                           frac=wbytes / sec / 1e9 / HBM_PEAK_GBS, traffic=MEASURED_TRAFFIC['moe_decode']),
             algorithmic_bytes=wbytes, active_experts=n_active, tflops=flops / sec / 1e12)
+    # the same layer with a shared expert (one more block-scaled MLP of inter 2048 on every token)
+    gen = torch.Generator(device=dev).manual_seed(20258)
+    sw13_q = (torch.randn(2 * I, H, device=dev, generator=gen) * (448 / H ** 0.5)).to(torch.float8_e4m3fn)
+    sw2_q = (torch.randn(H, I, device=dev, generator=gen) * (448 / I ** 0.5)).to(torch.float8_e4m3fn)
+    sw13_s = (0.5 + torch.rand(2 * I // 128, H // 128, device=dev, generator=gen)) / 448
+    sw2_s = (0.5 + torch.rand(H // 128, I // 128, device=dev, generator=gen)) / 448
+    del ws
+    ws2 = torch.empty(capi.moe_shared_workspace_bytes(T, H, I, I, E, k), dtype=torch.uint8, device=dev)
+    sec2 = timed_launches(
+        torch, lambda i: capi.moe_fp8_shared_launch(out, x, logits, w13_q, w13_s, w2_q, w2_s, sw13_q, sw13_s,
+                                                    sw2_q, sw2_s, ws2), steps, warmup)
+    flops2 = flops + T * (2 * H * 2 * I + 2 * I * H)
+    wbytes2 = wbytes + 3 * I * H + (3 * I * H // (128 * 128)) * 4
+    res['with_shared_expert'] = dict(
+        ms_per_step=sec2 * 1e3, unit=res['unit'],
+        value=flops2 / sec2 / 1e12 if prefill else wbytes2 / sec2 / 1e9,
+        note="moe_fp8_shared_launcher: the layer above plus one shared expert of inter 2048, seed 20258")
+    del ws2
     if cpu_baseline:
         n_tok = 4
         csec, n_used, cores = moe_cpu_baseline(torch, tensors, n_tok)
@@ -371,6 +389,10 @@ def main():
     }
     if 'cpu_baseline' in head:
         line["cpu_baseline"] = head['cpu_baseline']
+    shown = ('workload', 'value', 'unit', 'ms_per_step', 'dtype', 'roofline', 'cpu_baseline')
+    details = {k: v for k, v in head.items() if k not in shown}
+    if details:
+        line["details"] = details
     line["workloads"] = {k: v for k, v in results.items() if k != head_name}
     print(json.dumps(line))
 

@@ -32,6 +32,8 @@ SIGNATURES = {
     'sparse_mla_decode_num_splits': (c_int, [c_int, c_int, c_int, c_int]),
     'sparse_mla_decode_workspace_bytes': (c_size_t, [c_int, c_int, c_int, c_int]),
     'moe_route_launcher': (None, [_P, _P, _P, c_int, c_int, c_int, c_int, _P]),
+    'moe_route_grouped_launcher': (None, [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
+                                          c_int, _P]),
     'moe_sort_launcher': (None, [_P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P]),
     'moe_route_sort_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P]),
     'moe_quant_bf16_launcher': (None, [_P, _P, _P, c_int, c_int, c_int, _P]),
@@ -39,6 +41,10 @@ SIGNATURES = {
                                     c_int, _P]),
     'moe_down_launcher': (None, [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P]),
     'moe_combine_launcher': (None, [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P]),
+    'moe_combine_shared_launcher': (None, [_P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P]),
+    'moe_fp8_shared_workspace_bytes': (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
+    'moe_fp8_shared_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int,
+                                       c_int, c_int, c_int, c_int, c_int, c_int, _P]),
     'moe_fp8_workspace_bytes': (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
     'moe_fp8_workspace_layout': (None, [_P, c_int, c_int, c_int, c_int, c_int]),
     'moe_fp8_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int,
@@ -290,6 +296,27 @@ def moe_route_launch(ids, weights, logits, stream=None):
     return ids, weights
 
 
+def moe_route_grouped_launch(ids, weights, logits, bias, n_group, topk_group, normalise=True,
+                             routed_scaling_factor=1.0, stream=None):
+    """ids/weights [T, top_k] <- group-limited, bias-corrected top-k of logits [T, E] (bias [E] or None)."""
+    import torch
+    _device_contiguous(ids=ids, weights=weights, logits=logits)
+    T, E = logits.shape
+    top_k = ids.shape[1]
+    _require(ids.dtype == torch.int32 and weights.dtype == logits.dtype == torch.float32,
+             'moe_route_grouped: ids int32, weights/logits fp32')
+    _require(tuple(ids.shape) == tuple(weights.shape) == (T, top_k), 'moe_route_grouped: ids/weights shape')
+    if bias is not None:
+        _device_contiguous(bias=bias)
+        _require(bias.dtype == torch.float32 and tuple(bias.shape) == (E,), 'moe_route_grouped: bias fp32 [E]')
+    library().moe_route_grouped_launcher(_ptr(ids), _ptr(weights), _ptr(logits),
+                                         _ptr(bias) if bias is not None else c_void_p(None), T, E, top_k,
+                                         n_group, topk_group, 1 if normalise else 0,
+                                         float(routed_scaling_factor), 0, _stream(stream))
+    check_status('moe_route_grouped_launcher')
+    return ids, weights
+
+
 def moe_sort_launch(ids, n_experts, stream=None):
     """Returns (sorted_pairs, pair_pos, expert_offsets) int32 device tensors."""
     import torch
@@ -340,4 +367,38 @@ def moe_fp8_launch(out, x, logits, w13_q, w13_s, w2_q, w2_s, workspace, top_k=8,
                                T, H, I, E, top_k, 0 if out.dtype == torch.bfloat16 else 1, config,
                                _stream(stream))
     check_status('moe_fp8_launcher')
+    return out
+
+
+def moe_shared_workspace_bytes(tokens, hidden, inter, shared_inter, n_experts, top_k=8):
+    return int(library().moe_fp8_shared_workspace_bytes(tokens, hidden, inter, shared_inter, n_experts, top_k))
+
+
+def moe_fp8_shared_launch(out, x, logits, w13_q, w13_s, w2_q, w2_s, sw13_q, sw13_s, sw2_q, sw2_s, workspace,
+                          top_k=8, config=0, stream=None):
+    """The layer plus a shared expert (sw13_q [2*Is, H], sw13_s [2*Is/128, H/128], sw2_q [H, Is],
+    sw2_s [H/128, Is/128]) applied to every token with weight 1."""
+    import torch
+    _device_contiguous(out=out, x=x, logits=logits, w13_q=w13_q, w13_s=w13_s, w2_q=w2_q, w2_s=w2_s,
+                       sw13_q=sw13_q, sw13_s=sw13_s, sw2_q=sw2_q, sw2_s=sw2_s, workspace=workspace)
+    T, H = x.shape
+    E, I2, _ = w13_q.shape
+    I = I2 // 2
+    Is = sw13_q.shape[0] // 2
+    _require(x.dtype == torch.bfloat16 and logits.dtype == torch.float32, 'moe_fp8: x bf16, logits fp32')
+    _require(out.dtype in (torch.bfloat16, torch.float32) and tuple(out.shape) == (T, H), 'moe_fp8: out')
+    _require(all(t.element_size() == 1 for t in (w13_q, w2_q, sw13_q, sw2_q)), 'moe_fp8: weights must be e4m3')
+    _require(tuple(w13_q.shape) == (E, 2 * I, H) and tuple(w2_q.shape) == (E, H, I), 'moe_fp8: weight shapes')
+    _require(tuple(w13_s.shape) == (E, 2 * I // 128, H // 128) and tuple(w2_s.shape) == (E, H // 128, I // 128),
+             'moe_fp8: scale shapes')
+    _require(tuple(sw13_q.shape) == (2 * Is, H) and tuple(sw2_q.shape) == (H, Is), 'moe_fp8: shared weight shapes')
+    _require(tuple(sw13_s.shape) == (2 * Is // 128, H // 128) and tuple(sw2_s.shape) == (H // 128, Is // 128),
+             'moe_fp8: shared scale shapes')
+    _require(all(t.dtype == torch.float32 for t in (w13_s, w2_s, sw13_s, sw2_s)), 'moe_fp8: scales fp32')
+    _require(tuple(logits.shape) == (T, E), 'moe_fp8: logits shape')
+    library().moe_fp8_shared_launcher(
+        _ptr(out), _ptr(x), _ptr(logits), _ptr(w13_q), _ptr(w13_s), _ptr(w2_q), _ptr(w2_s), _ptr(sw13_q),
+        _ptr(sw13_s), _ptr(sw2_q), _ptr(sw2_s), _ptr(workspace), workspace.numel() * workspace.element_size(),
+        T, H, I, Is, E, top_k, 0 if out.dtype == torch.bfloat16 else 1, config, _stream(stream))
+    check_status('moe_fp8_shared_launcher')
     return out

@@ -46,12 +46,26 @@ using namespace moe;
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 
-// out[t, :] = sum_k weights[t, k] * y[pair_pos[t*top_k + k], :], k ascending, fp32.
+// the "sort" of a single expert that takes every token once: identity order, offsets {0, tokens}
+__global__ __launch_bounds__(256) void moe_identity_sort_kernel(int* __restrict__ sorted_pairs,
+                                                                int* __restrict__ pair_pos,
+                                                                int* __restrict__ expert_offsets,
+                                                                int tokens) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < tokens) {
+        sorted_pairs[i] = i;
+        pair_pos[i] = i;
+    }
+    if (i < 2) expert_offsets[i] = i * tokens;
+}
+
+// out[t, :] = sum_k weights[t, k] * y[pair_pos[t*top_k + k], :] (k ascending) + y_shared[t, :], fp32.
 // blockIdx.x is the token, blockIdx.y a 1024-column slice; 4 columns per lane.
 template <typename OUT>
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y,
                                                           const float* __restrict__ weights,
                                                           const int* __restrict__ pair_pos,
+                                                          const float* __restrict__ y_shared,
                                                           OUT* __restrict__ out, int hidden,
                                                           int top_k) {
     const int t = blockIdx.x;
@@ -73,6 +87,9 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
                 if (k0 + j < top_k) acc += v[j] * w[j];
             }
         }
+        // the shared expert's row, if there is one, is added last
+        if (y_shared != nullptr)
+            acc += __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(y_shared + (size_t)t * hidden + c));
         OUT* dst = out + (size_t)t * hidden + c;
         if constexpr (sizeof(OUT) == 4) {
             *reinterpret_cast<floatx4*>(dst) = acc;
@@ -86,10 +103,12 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
 }  // namespace
 
 // out [tokens, hidden] (bf16 if out_dtype == 0, fp32 if 1) from y [tokens*top_k, hidden] fp32 in
-// sorted order, weights [tokens, top_k], pair_pos [tokens*top_k].
-extern "C" void moe_combine_launcher(void* out, const float* y, const float* weights,
-                                     const int* pair_pos, int tokens, int hidden, int top_k,
-                                     int out_dtype, int config, hipStream_t stream) {
+// sorted order, weights [tokens, top_k], pair_pos [tokens*top_k]; y_shared [tokens, hidden] fp32
+// (or null) is added to every token's sum last.
+extern "C" void moe_combine_shared_launcher(void* out, const float* y, const float* weights,
+                                            const int* pair_pos, const float* y_shared, int tokens,
+                                            int hidden, int top_k, int out_dtype, int config,
+                                            hipStream_t stream) {
     (void)config;
     if (tokens <= 0) return;
     if (hidden <= 0 || hidden % 4 != 0 || top_k <= 0 || (out_dtype != 0 && out_dtype != 1)) {
@@ -97,18 +116,25 @@ extern "C" void moe_combine_launcher(void* out, const float* y, const float* wei
         return;
     }
     if (!out || !y || !weights || !pair_pos || (reinterpret_cast<uintptr_t>(y) & 15u) ||
-        (reinterpret_cast<uintptr_t>(out) & 15u)) {
+        (reinterpret_cast<uintptr_t>(out) & 15u) || (reinterpret_cast<uintptr_t>(y_shared) & 15u)) {
         caa::set_status(CAA_BAD_ARGUMENT);
         return;
     }
     const dim3 grid(tokens, (hidden + 1023) / 1024);
     if (out_dtype == 0) {
-        moe_combine_kernel<__bf16><<<grid, 256, 0, stream>>>(y, weights, pair_pos,
+        moe_combine_kernel<__bf16><<<grid, 256, 0, stream>>>(y, weights, pair_pos, y_shared,
                                                             static_cast<__bf16*>(out), hidden, top_k);
     } else {
-        moe_combine_kernel<float><<<grid, 256, 0, stream>>>(y, weights, pair_pos,
+        moe_combine_kernel<float><<<grid, 256, 0, stream>>>(y, weights, pair_pos, y_shared,
                                                            static_cast<float*>(out), hidden, top_k);
     }
+}
+
+extern "C" void moe_combine_launcher(void* out, const float* y, const float* weights,
+                                     const int* pair_pos, int tokens, int hidden, int top_k,
+                                     int out_dtype, int config, hipStream_t stream) {
+    moe_combine_shared_launcher(out, y, weights, pair_pos, nullptr, tokens, hidden, top_k, out_dtype,
+                                config, stream);
 }
 
 extern "C" size_t moe_fp8_workspace_bytes(int tokens, int hidden, int inter, int n_experts,
@@ -129,35 +155,13 @@ extern "C" void moe_fp8_workspace_layout(size_t* offsets10, int tokens, int hidd
     for (int i = 0; i < 10; ++i) offsets10[i] = static_cast<const char*>(ptrs[i]) - base;
 }
 
-// The whole layer. out [tokens, hidden] bf16 (out_dtype 0) or fp32 (out_dtype 1).
-// config: 0 = choose by the average number of pairs per expert (above 32: LDS-tiled GEMMs, else
-// weight streaming); 16 forces the tiled GEMMs; 1, 2, 4 (+8) force streaming, see moe_gate_up_launcher.
-extern "C" void moe_fp8_launcher(void* out, const void* x, const float* logits, const void* w13_q,
-                                 const float* w13_s, const void* w2_q, const float* w2_s,
-                                 void* workspace, size_t workspace_bytes, int tokens, int hidden,
-                                 int inter, int n_experts, int top_k, int out_dtype, int config,
-                                 hipStream_t stream) {
-    if (tokens <= 0) return;
-    if (hidden <= 0 || inter <= 0 || hidden % GROUP != 0 || inter % GROUP != 0 || n_experts <= 0 ||
-        n_experts > 512 || top_k <= 0 || top_k > 64 || top_k > n_experts ||
-        (long)tokens * top_k > 0x7fffffffL / 4 || (out_dtype != 0 && out_dtype != 1)) {
-        caa::set_status(CAA_UNSUPPORTED_SHAPE);
-        return;
-    }
-    if (!out || !x || !logits || !w13_q || !w13_s || !w2_q || !w2_s || !workspace ||
-        (reinterpret_cast<uintptr_t>(workspace) & 255u)) {
-        caa::set_status(CAA_BAD_ARGUMENT);
-        return;
-    }
-    const moe::Workspace w = moe::carve_workspace(workspace, tokens, hidden, inter, n_experts, top_k);
-    if (workspace_bytes < w.bytes) {
-        caa::set_status(CAA_WORKSPACE_TOO_SMALL);
-        return;
-    }
-    moe_route_sort_launcher(w.ids, w.weights, w.sorted_pairs, w.pair_pos, w.expert_offsets, w.chunk_hist,
-                            logits, tokens, n_experts, top_k, 0, stream);
-    moe_quant_bf16_launcher(w.x_q, w.x_s, x, tokens, hidden, 0, stream);
-    // Many pairs per expert: LDS-tiled GEMMs (256 x 256 tiles). Few: the weight-streaming form.
+namespace {
+
+// gate/up and down GEMMs of the experts over the quantised activations and the sort in `w`; result
+// in w.y. Many pairs per expert: LDS-tiled GEMMs (256 x 256 tiles). Few: the weight-streaming form.
+void run_expert_gemms(const moe::Workspace& w, const void* w13_q, const float* w13_s,
+                      const void* w2_q, const float* w2_s, int tokens, int hidden, int inter,
+                      int n_experts, int top_k, int config, hipStream_t stream) {
     // (the tiled kernels address activations with 32-bit byte offsets)
     const bool fits32 = (unsigned long long)tokens * hidden < (1ull << 32) &&
                         (unsigned long long)tokens * top_k * inter < (1ull << 32);
@@ -177,5 +181,96 @@ extern "C" void moe_fp8_launcher(void* out, const void* x, const float* logits, 
         moe_down_launcher(w.y, w.h_q, w.h_s, w2_q, w2_s, w.expert_offsets, tokens, hidden, inter,
                           n_experts, top_k, config, stream);
     }
+}
+
+bool layer_shape_ok(int hidden, int inter, int n_experts, int top_k, int tokens, int out_dtype) {
+    return hidden > 0 && inter > 0 && hidden % GROUP == 0 && inter % GROUP == 0 && n_experts > 0 &&
+           n_experts <= 512 && top_k > 0 && top_k <= 64 && top_k <= n_experts &&
+           (long)tokens * top_k <= 0x7fffffffL / 4 && (out_dtype == 0 || out_dtype == 1);
+}
+
+}  // namespace
+
+// The whole layer. out [tokens, hidden] bf16 (out_dtype 0) or fp32 (out_dtype 1).
+// config: 0 = choose by the average number of pairs per expert (above 32: LDS-tiled GEMMs, else
+// weight streaming); 16 forces the tiled GEMMs; 1, 2, 4 (+8) force streaming, see moe_gate_up_launcher.
+extern "C" void moe_fp8_launcher(void* out, const void* x, const float* logits, const void* w13_q,
+                                 const float* w13_s, const void* w2_q, const float* w2_s,
+                                 void* workspace, size_t workspace_bytes, int tokens, int hidden,
+                                 int inter, int n_experts, int top_k, int out_dtype, int config,
+                                 hipStream_t stream) {
+    if (tokens <= 0) return;
+    if (!layer_shape_ok(hidden, inter, n_experts, top_k, tokens, out_dtype)) {
+        caa::set_status(CAA_UNSUPPORTED_SHAPE);
+        return;
+    }
+    if (!out || !x || !logits || !w13_q || !w13_s || !w2_q || !w2_s || !workspace ||
+        (reinterpret_cast<uintptr_t>(workspace) & 255u)) {
+        caa::set_status(CAA_BAD_ARGUMENT);
+        return;
+    }
+    const moe::Workspace w = moe::carve_workspace(workspace, tokens, hidden, inter, n_experts, top_k);
+    if (workspace_bytes < w.bytes) {
+        caa::set_status(CAA_WORKSPACE_TOO_SMALL);
+        return;
+    }
+    moe_route_sort_launcher(w.ids, w.weights, w.sorted_pairs, w.pair_pos, w.expert_offsets, w.chunk_hist,
+                            logits, tokens, n_experts, top_k, 0, stream);
+    moe_quant_bf16_launcher(w.x_q, w.x_s, x, tokens, hidden, 0, stream);
+    run_expert_gemms(w, w13_q, w13_s, w2_q, w2_s, tokens, hidden, inter, n_experts, top_k, config, stream);
     moe_combine_launcher(out, w.y, w.weights, w.pair_pos, tokens, hidden, top_k, out_dtype, 0, stream);
+}
+
+// Workspace of moe_fp8_shared_launcher: the routed experts' workspace followed by the same
+// structure for one expert that takes every token once.
+extern "C" size_t moe_fp8_shared_workspace_bytes(int tokens, int hidden, int inter, int shared_inter,
+                                                 int n_experts, int top_k) {
+    if (tokens <= 0 || hidden <= 0 || inter <= 0 || shared_inter <= 0 || n_experts <= 0 || top_k <= 0)
+        return 0;
+    return moe::carve_workspace(nullptr, tokens, hidden, inter, n_experts, top_k).bytes +
+           moe::carve_workspace(nullptr, tokens, hidden, shared_inter, 1, 1).bytes;
+}
+
+// The layer with a shared expert: out = sum_k w[t,k] * expert_k(x[t]) + shared(x[t]), where the
+// shared expert is one more block-scaled MLP (sw13_q [2*shared_inter, hidden], sw13_s
+// [2*shared_inter/128, hidden/128], sw2_q [hidden, shared_inter], sw2_s [hidden/128,
+// shared_inter/128]) applied to every token with weight 1. It runs through the same kernels as
+// the routed experts (as a group of one expert holding all tokens, on the activations quantised
+// once for both) and its fp32 row is added last in the combine.
+extern "C" void moe_fp8_shared_launcher(void* out, const void* x, const float* logits,
+                                        const void* w13_q, const float* w13_s, const void* w2_q,
+                                        const float* w2_s, const void* sw13_q, const float* sw13_s,
+                                        const void* sw2_q, const float* sw2_s, void* workspace,
+                                        size_t workspace_bytes, int tokens, int hidden, int inter,
+                                        int shared_inter, int n_experts, int top_k, int out_dtype,
+                                        int config, hipStream_t stream) {
+    if (tokens <= 0) return;
+    if (!layer_shape_ok(hidden, inter, n_experts, top_k, tokens, out_dtype) || shared_inter <= 0 ||
+        shared_inter % GROUP != 0) {
+        caa::set_status(CAA_UNSUPPORTED_SHAPE);
+        return;
+    }
+    if (!out || !x || !logits || !w13_q || !w13_s || !w2_q || !w2_s || !sw13_q || !sw13_s || !sw2_q ||
+        !sw2_s || !workspace || (reinterpret_cast<uintptr_t>(workspace) & 255u)) {
+        caa::set_status(CAA_BAD_ARGUMENT);
+        return;
+    }
+    const moe::Workspace w = moe::carve_workspace(workspace, tokens, hidden, inter, n_experts, top_k);
+    moe::Workspace sh = moe::carve_workspace(static_cast<char*>(workspace) + w.bytes, tokens, hidden,
+                                             shared_inter, 1, 1);
+    if (workspace_bytes < w.bytes + sh.bytes) {
+        caa::set_status(CAA_WORKSPACE_TOO_SMALL);
+        return;
+    }
+    moe_route_sort_launcher(w.ids, w.weights, w.sorted_pairs, w.pair_pos, w.expert_offsets, w.chunk_hist,
+                            logits, tokens, n_experts, top_k, 0, stream);
+    moe_quant_bf16_launcher(w.x_q, w.x_s, x, tokens, hidden, 0, stream);
+    run_expert_gemms(w, w13_q, w13_s, w2_q, w2_s, tokens, hidden, inter, n_experts, top_k, config, stream);
+    sh.x_q = w.x_q;
+    sh.x_s = w.x_s;
+    moe_identity_sort_kernel<<<(tokens + 255) / 256, 256, 0, stream>>>(sh.sorted_pairs, sh.pair_pos,
+                                                                      sh.expert_offsets, tokens);
+    run_expert_gemms(sh, sw13_q, sw13_s, sw2_q, sw2_s, tokens, hidden, shared_inter, 1, 1, config, stream);
+    moe_combine_shared_launcher(out, w.y, w.weights, w.pair_pos, sh.y, tokens, hidden, top_k, out_dtype,
+                                0, stream);
 }

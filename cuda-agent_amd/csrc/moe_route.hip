@@ -73,6 +73,105 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     }
 }
 
+// Group-limited routing with a selection bias (the DeepSeek-V3 router): one wavefront per token.
+//   score = sigmoid(logit);  choice = score + bias
+//   group value = sum of the 2 largest choice values of the group (groups are runs of
+//                 n_experts / n_group consecutive experts)
+//   the topk_group groups with the largest value stay (ties to the lower group), the others are out
+//   ids = the top_k largest choice values among the experts that stay, descending, ties to the
+//         lower expert id
+//   weights = score[ids] (the unbiased score), divided by their sum + 1e-20 if normalise, times scale
+// LDS per wavefront: the token's choice values and scores, n_experts floats each.
+template <int PER_LANE>
+__global__ __launch_bounds__(256) void moe_route_grouped_kernel(
+    const float* __restrict__ logits, const float* __restrict__ bias, int* __restrict__ ids,
+    float* __restrict__ weights, int tokens, int n_experts, int top_k, int n_group, int topk_group,
+    int normalise, float scale) {
+    extern __shared__ float s_route[];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int t = blockIdx.x * 4 + wave;
+    if (t >= tokens) return;  // (no workgroup barrier below: a wavefront only reads what it wrote)
+    float* s_choice = s_route + (size_t)wave * 2 * n_experts;
+    float* s_score = s_choice + n_experts;
+    const int group_size = n_experts / n_group;
+
+    float choice[PER_LANE];
+#pragma unroll
+    for (int j = 0; j < PER_LANE; ++j) {
+        const int e = j * 64 + lane;
+        choice[j] = -INFINITY;
+        if (e < n_experts) {
+            const float score = 1.f / (1.f + expf(-logits[(size_t)t * n_experts + e]));
+            choice[j] = score + (bias != nullptr ? bias[e] : 0.f);
+            s_choice[e] = choice[j];
+            s_score[e] = score;
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+
+    // lane g: value of group g
+    float value = -INFINITY;
+    if (lane < n_group) {
+        float first = -INFINITY, second = -INFINITY;
+        for (int i = 0; i < group_size; ++i) {
+            const float c = s_choice[lane * group_size + i];
+            if (c > first) {
+                second = first;
+                first = c;
+            } else if (c > second) {
+                second = c;
+            }
+        }
+        value = group_size > 1 ? first + second : first;
+    }
+    // rank of group `lane` among the groups; the topk_group best stay
+    int better = 0;
+    for (int g = 0; g < n_group; ++g) {
+        const float other = __shfl(value, g);
+        better += (other > value || (other == value && g < lane)) ? 1 : 0;
+    }
+    const unsigned long long stay_mask = __ballot(lane < n_group && better < topk_group);
+
+    unsigned long long key[PER_LANE];
+#pragma unroll
+    for (int j = 0; j < PER_LANE; ++j) {
+        const int e = j * 64 + lane;
+        const bool stays = e < n_experts && ((stay_mask >> (e / group_size)) & 1ull);
+        key[j] = stays ? rank_key(choice[j], e) : 0ull;
+    }
+    float my_score = 0.f;  // lane k keeps the k-th choice
+    int my_id = 0;
+    float total = 0.f;
+    for (int k = 0; k < top_k; ++k) {
+        unsigned long long best = 0ull;
+#pragma unroll
+        for (int j = 0; j < PER_LANE; ++j) best = key[j] > best ? key[j] : best;
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            const unsigned long long other = __shfl_xor(best, off);
+            best = other > best ? other : best;
+        }
+        const int id = 0x7fffffff - (int)(unsigned)(best & 0xffffffffull);
+#pragma unroll
+        for (int j = 0; j < PER_LANE; ++j) {
+            if (j * 64 + lane == id) key[j] = 0ull;  // taken
+        }
+        const float score = s_score[id];
+        total += score;
+        if (lane == k) {
+            my_score = score;
+            my_id = id;
+        }
+    }
+    if (lane < top_k) {
+        ids[(size_t)t * top_k + lane] = my_id;
+        const float w = normalise ? my_score / (total + 1e-20f) : my_score;
+        weights[(size_t)t * top_k + lane] = w * scale;
+    }
+}
+
 // chunk_hist[chunk][e] = number of pairs of chunk `chunk` routed to expert e
 __global__ __launch_bounds__(256) void moe_hist_kernel(const int* __restrict__ ids,
                                                        int* __restrict__ chunk_hist, int pairs,
@@ -340,6 +439,39 @@ extern "C" void moe_route_launcher(int* ids, float* weights, const float* logits
         moe_route_kernel<4><<<blocks, 256, 0, stream>>>(logits, ids, weights, tokens, n_experts, top_k);
     } else {
         moe_route_kernel<8><<<blocks, 256, 0, stream>>>(logits, ids, weights, tokens, n_experts, top_k);
+    }
+}
+
+// Group-limited routing with a selection bias (see moe_route_grouped_kernel).
+// bias [n_experts] fp32 or null. n_experts a multiple of n_group, n_group <= 64,
+// topk_group <= n_group, top_k <= topk_group * (n_experts / n_group).
+extern "C" void moe_route_grouped_launcher(int* ids, float* weights, const float* logits,
+                                           const float* bias, int tokens, int n_experts, int top_k,
+                                           int n_group, int topk_group, int normalise,
+                                           float routed_scaling_factor, int config,
+                                           hipStream_t stream) {
+    (void)config;
+    if (tokens <= 0) return;
+    if (n_experts <= 0 || n_experts > 512 || top_k <= 0 || top_k > 64 || n_group <= 0 ||
+        n_group > 64 || n_experts % n_group != 0 || topk_group <= 0 || topk_group > n_group ||
+        (long long)topk_group * (n_experts / n_group) < top_k) {
+        caa::set_status(CAA_UNSUPPORTED_SHAPE);
+        return;
+    }
+    if (!ids || !weights || !logits) {
+        caa::set_status(CAA_BAD_ARGUMENT);
+        return;
+    }
+    const int blocks = (tokens + 3) / 4;
+    const size_t lds = (size_t)4 * 2 * n_experts * sizeof(float);
+    if (n_experts <= 256) {
+        moe_route_grouped_kernel<4><<<blocks, 256, lds, stream>>>(
+            logits, bias, ids, weights, tokens, n_experts, top_k, n_group, topk_group, normalise,
+            routed_scaling_factor);
+    } else {
+        moe_route_grouped_kernel<8><<<blocks, 256, lds, stream>>>(
+            logits, bias, ids, weights, tokens, n_experts, top_k, n_group, topk_group, normalise,
+            routed_scaling_factor);
     }
 }
 

@@ -167,6 +167,20 @@ size_t sparse_mla_decode_workspace_bytes(int batch, int n_heads, int topk, int c
 void moe_route_launcher(int* ids, float* weights, const float* logits, int tokens, int n_experts,
                         int top_k, int config, hipStream_t stream);
 
+/* Group-limited routing with a selection bias, the router of DeepSeek-V3-style layers (caller-
+ * side neighbour of moe_route_launcher; same launcher pattern):
+ *   score = sigmoid(logit), choice = score + bias; a group (n_experts/n_group consecutive
+ *   experts) is valued by the sum of its 2 largest choice values; only the topk_group best groups
+ *   stay (ties to the lower group); ids = the top_k largest choice values among the experts that
+ *   stay, descending, ties to the lower expert id; weights = score[ids], divided by their sum +
+ *   1e-20 if normalise != 0, times routed_scaling_factor.
+ * bias [n_experts] fp32 or NULL. n_experts <= 512 and a multiple of n_group, n_group <= 64,
+ * topk_group <= n_group, top_k <= min(64, topk_group * n_experts / n_group). */
+void moe_route_grouped_launcher(int* ids, float* weights, const float* logits, const float* bias,
+                                int tokens, int n_experts, int top_k, int n_group, int topk_group,
+                                int normalise, float routed_scaling_factor, int config,
+                                hipStream_t stream);
+
 /* Stable counting sort of the tokens*top_k (token, slot) pairs by expert id:
  * sorted_pairs[pos] = token*top_k + slot, pair_pos = its inverse, expert e owns positions
  * expert_offsets[e] .. expert_offsets[e+1]-1 (expert_offsets has n_experts+1 entries).
@@ -225,6 +239,30 @@ void moe_fp8_launcher(void* out, const void* x, const float* logits, const void*
                       const float* w13_s, const void* w2_q, const float* w2_s, void* workspace,
                       size_t workspace_bytes, int tokens, int hidden, int inter, int n_experts,
                       int top_k, int out_dtype, int config, hipStream_t stream);
+
+/* The same sum with one more fp32 row per token added last: y_shared [tokens, hidden] (the shared
+ * expert's output) or NULL. */
+void moe_combine_shared_launcher(void* out, const float* y, const float* weights,
+                                 const int* pair_pos, const float* y_shared, int tokens, int hidden,
+                                 int top_k, int out_dtype, int config, hipStream_t stream);
+
+/* The layer with a shared expert (the caller-side neighbour of moe_fp8_launcher in
+ * DeepSeek-V3-style layers; same launcher pattern): out = sum_k w[t,k] * expert_k(x[t]) +
+ * shared(x[t]). The shared expert is one more block-scaled MLP, sw13_q [2*shared_inter, hidden],
+ * sw13_s [2*shared_inter/128, hidden/128], sw2_q [hidden, shared_inter], sw2_s [hidden/128,
+ * shared_inter/128], applied to every token with weight 1 on the activations quantised once for
+ * both; its fp32 row is added after the routed experts' weighted sum. workspace:
+ * moe_fp8_shared_workspace_bytes(...) bytes, 256-byte aligned; its first
+ * moe_fp8_workspace_bytes(...) bytes have the layout moe_fp8_workspace_layout describes.
+ * Everything else as moe_fp8_launcher. */
+size_t moe_fp8_shared_workspace_bytes(int tokens, int hidden, int inter, int shared_inter,
+                                      int n_experts, int top_k);
+void moe_fp8_shared_launcher(void* out, const void* x, const float* logits, const void* w13_q,
+                             const float* w13_s, const void* w2_q, const float* w2_s,
+                             const void* sw13_q, const float* sw13_s, const void* sw2_q,
+                             const float* sw2_s, void* workspace, size_t workspace_bytes, int tokens,
+                             int hidden, int inter, int shared_inter, int n_experts, int top_k,
+                             int out_dtype, int config, hipStream_t stream);
 
 #ifdef __cplusplus
 }

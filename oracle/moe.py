@@ -21,6 +21,16 @@ Ranking by logit equals ranking by an exact sigmoid and does not depend on how a
 sigmoid implementation rounds. The reference repository has no implementation of this operator;
 only its model contract (agent_workdir/model.py:9-26) shapes the functions below.
 
+``route_grouped`` is the router a DeepSeek-V3-style layer uses in place of ``route`` (group-limited
+choice with a selection bias; no counterpart in the reference repository). Pinned by scalar loops
+on small sizes, by the reduction to ``route`` when there is one group and no bias, by its
+invariants (chosen experts lie in exactly topk_group groups, weights sum to the scaling factor),
+and by a golden fixture written from the third-party ``transformers`` router
+(tests/golden/make_router_golden.py).
+
+``moe_forward_shared`` adds the shared expert of such a layer; it is built from ``moe_forward`` itself
+and pinned by a float64 dense evaluation of the same sum on a tiny shape.
+
 Pinned by (tests/test_oracle_moe.py):
   * e4m3: the 256-entry decode table against torch's float8_e4m3fn and the closed form; the
     encoder against torch's cast on every representable value, every midpoint and random
@@ -112,6 +122,29 @@ def route(logits, top_k=8):
     return order.int(), score / score.sum(dim=-1, keepdim=True)
 
 
+def route_grouped(logits, bias, top_k, n_group, topk_group, normalise=True, routed_scaling_factor=1.0):
+    """Group-limited routing with a selection bias.
+
+    score = sigmoid(logits); choice = score + bias. A group is a run of E/n_group consecutive experts and
+    is valued by the sum of its 2 largest choice values; the topk_group best groups stay (ties to the lower
+    group). ids int32 [T,k]: the top_k largest choice values among the experts that stay, descending, ties
+    to the lower id. weights fp32 [T,k] = score[ids] (/ (sum + 1e-20) if ``normalise``) * scaling factor.
+    Returns (ids, weights, choice) - ``choice`` fp32 [T,E] lets a checker see how close a decision was."""
+    T, E = logits.shape
+    score = torch.sigmoid(logits.float())
+    choice = score if bias is None else score + bias.float()[None]
+    grouped = choice.view(T, n_group, E // n_group)
+    value = grouped.topk(min(2, E // n_group), dim=-1).values.sum(dim=-1)
+    stay_groups = torch.sort(value, dim=-1, descending=True, stable=True).indices[:, :topk_group]
+    stay = torch.zeros(T, n_group, dtype=torch.bool).scatter_(1, stay_groups, True)
+    masked = grouped.masked_fill(~stay[:, :, None], float('-inf')).reshape(T, E)
+    ids = torch.sort(masked, dim=-1, descending=True, stable=True).indices[:, :top_k]
+    w = score.gather(1, ids)
+    if normalise:
+        w = w / (w.sum(dim=-1, keepdim=True) + 1e-20)
+    return ids.int(), w * routed_scaling_factor, choice
+
+
 def sort_pairs(ids, n_experts):
     """Stable counting sort of the flattened (token, slot) pairs by expert.
     Returns sorted_pairs int32 [T*k] (flat pair index at each sorted position),
@@ -159,6 +192,18 @@ def moe_forward(x, logits, w13_q, w13_s, w2_q, w2_s, top_k=8, out_dtype=torch.bf
     if return_intermediates:
         return out, dict(ids=ids, weights=weights, x_q=x_q, x_s=x_s, h_q=h_q_all, h_s=h_s_all, y=y)
     return out
+
+
+def moe_forward_shared(x, logits, w13_q, w13_s, w2_q, w2_s, sw13_q, sw13_s, sw2_q, sw2_s, top_k=8,
+                       out_dtype=torch.bfloat16):
+    """The layer plus a shared expert: one more block-scaled MLP (sw13_q [2*Is,H], sw13_s, sw2_q [H,Is],
+    sw2_s) applied to every token with weight 1, added in fp32 after the routed experts' weighted sum.
+    The shared expert is evaluated by the same stage functions: a layer of one expert chosen by every
+    token with routing weight s/s = 1."""
+    routed = moe_forward(x, logits, w13_q, w13_s, w2_q, w2_s, top_k, torch.float32)
+    shared = moe_forward(x, torch.zeros(x.shape[0], 1), sw13_q[None], sw13_s[None], sw2_q[None], sw2_s[None],
+                         1, torch.float32)
+    return (routed + shared).to(out_dtype)
 
 
 # ---------------------------------------------------------------------------- synthetic inputs

@@ -1,0 +1,77 @@
+"""The MoE layer with a shared expert, through the C ABI.
+
+The shared expert runs through the same kernels as the routed experts (a group of one expert that holds every
+token), so the bar has two parts. Bit-equality with already-checked paths: the fp32 output must equal the fp32
+output of the routed layer plus the fp32 output of a one-expert layer over the shared weights, added in that
+order; the bf16 output must be the rounding of the fp32 one. And the end-to-end bounds of the layer against the
+oracle: rms error <= 0.5 %, at most 1 output in 1000 beyond 2e-2 rms (isolated requantised codes land on the
+other side of a rounding boundary on this hardware path), none beyond 0.15 rms."""
+import pytest
+import torch
+
+from oracle import moe
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-2
+
+
+def make_case(dev, T, H, I, Is, E, seed):
+    gen = torch.Generator().manual_seed(seed)
+    w = moe.moe_make_weights(E, H, I, gen)
+    sw = tuple(t[0].contiguous() for t in moe.moe_make_weights(1, H, Is, gen))
+    x, logits = moe.moe_make_inputs(T, H, E, gen)
+    return x, logits, w, sw, [t.to(dev) for t in (x, logits, *w, *sw)]
+
+
+def run_shared(capi, dts, top_k, config=0, dtype=torch.bfloat16):
+    x, logits, w13_q, w13_s, w2_q, w2_s, sw13_q, sw13_s, sw2_q, sw2_s = dts
+    T, H = x.shape
+    E, I2, _ = w13_q.shape
+    ws = torch.empty(capi.moe_shared_workspace_bytes(T, H, I2 // 2, sw13_q.shape[0] // 2, E, top_k),
+                     dtype=torch.uint8, device=x.device)
+    out = torch.full((T, H), float('nan'), dtype=dtype, device=x.device)
+    capi.moe_fp8_shared_launch(out, *dts, ws, top_k=top_k, config=config)
+    torch.cuda.synchronize()
+    return out
+
+
+def run_plain(capi, x, logits, w13_q, w13_s, w2_q, w2_s, top_k, config):
+    T, H = x.shape
+    E, I2, _ = w13_q.shape
+    ws = torch.empty(capi.moe_workspace_bytes(T, H, I2 // 2, E, top_k), dtype=torch.uint8, device=x.device)
+    out = torch.full((T, H), float('nan'), dtype=torch.float32, device=x.device)
+    capi.moe_fp8_launch(out, x, logits, w13_q, w13_s, w2_q, w2_s, ws, top_k=top_k, config=config)
+    torch.cuda.synchronize()
+    return out
+
+
+@pytest.mark.parametrize('config', [0, 4, 16])
+@pytest.mark.parametrize('shape', [(64, 512, 256, 256, 16, 4), (300, 256, 128, 384, 8, 2), (1, 256, 128, 128, 4, 1),
+                                   (1100, 512, 256, 128, 5, 2), (33, 768, 384, 256, 40, 8)])
+def test_shared_layer(capi, dev, shape, config):
+    T, H, I, Is, E, k = shape
+    x, logits, w, sw, dts = make_case(dev, T, H, I, Is, E, 3000 + T)
+    exact = run_shared(capi, dts, k, config, torch.float32)
+    assert torch.isfinite(exact).all()
+    # the same kernels, called as two layers
+    routed = run_plain(capi, *dts[:6], k, config)
+    zeros = torch.zeros(T, 1, device=dev)
+    shared = run_plain(capi, dts[0], zeros, *(t[None] for t in dts[6:]), 1, config)
+    assert torch.equal(exact, routed + shared)
+    assert torch.equal(run_shared(capi, dts, k, config), exact.bfloat16())
+    # against the oracle
+    ref = moe.moe_forward_shared(x, logits, *w, *sw, top_k=k, out_dtype=torch.float32)
+    rms = ref.double().pow(2).mean().sqrt()
+    diff = (exact.cpu() - ref).double().abs()
+    assert (diff.pow(2).mean().sqrt() / rms).item() <= 5e-3
+    assert (diff > TOL * rms).double().mean().item() <= 1e-3
+    assert (diff.max() / rms).item() <= 0.15
+
+
+def test_rejects_bad_arguments(capi, dev):
+    x, logits, w, sw, dts = make_case(dev, 8, 256, 128, 128, 4, 1)
+    out = torch.empty(8, 256, dtype=torch.bfloat16, device=dev)
+    small = torch.empty(capi.moe_workspace_bytes(8, 256, 128, 4, 2), dtype=torch.uint8, device=dev)
+    with pytest.raises(capi.LaunchRejected):          # the routed layer's workspace is not enough
+        capi.moe_fp8_shared_launch(out, *dts, small, top_k=2)
+    torch.cuda.synchronize()

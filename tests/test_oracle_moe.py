@@ -172,3 +172,104 @@ def test_weight_generator_has_no_nan_codes():
         assert ((q.view(torch.uint8) & 0x7F) != 0x7F).all()
     assert (w13_s > 0.5 / 448 - 1e-9).all() and (w13_s < 1.5 / 448 + 1e-9).all()
     assert w13_s.shape == (2, 2, 2) and w2_s.shape == (2, 2, 1)
+
+
+# ---- group-limited routing with a selection bias -------------------------------------------------
+
+def _route_grouped_loops(logits, bias, top_k, n_group, topk_group, normalise, scale):
+    T, E = logits.shape
+    gs = E // n_group
+    ids, weights = [], []
+    for t in range(T):
+        score = [float(torch.sigmoid(logits[t, e])) for e in range(E)]
+        choice = [float(np.float32(score[e]) + np.float32(0.0 if bias is None else float(bias[e]))) for e in range(E)]
+        value = []
+        for g in range(n_group):
+            best = sorted(choice[g * gs:(g + 1) * gs], reverse=True)[:2]
+            value.append(float(np.float32(sum(np.float32(b) for b in best))))
+        groups = sorted(range(n_group), key=lambda g: (-value[g], g))[:topk_group]
+        candidates = [e for e in range(E) if e // gs in groups]
+        chosen = sorted(candidates, key=lambda e: (-choice[e], e))[:top_k]
+        w = np.array([score[e] for e in chosen], dtype=np.float32)
+        if normalise:
+            w = w / (w.sum(dtype=np.float32) + np.float32(1e-20))
+        ids.append(chosen)
+        weights.append(w * np.float32(scale))
+    return np.array(ids), np.array(weights)
+
+
+@pytest.mark.parametrize('shape', [(7, 16, 3, 4, 2, True, 1.0), (5, 64, 8, 8, 4, True, 2.5), (6, 32, 4, 4, 4, False, 1.0),
+                                   (4, 24, 5, 3, 2, True, 0.5), (3, 8, 2, 8, 3, True, 1.0)])
+def test_grouped_routing_matches_scalar_loops(shape):
+    T, E, k, G, kg, norm, scale = shape
+    gen = torch.Generator().manual_seed(T * 100 + E)
+    logits = torch.randn(T, E, generator=gen)
+    bias = 0.2 * torch.randn(E, generator=gen)
+    ids, w, _ = moe.route_grouped(logits, bias, k, G, kg, norm, scale)
+    want_ids, want_w = _route_grouped_loops(logits, bias, k, G, kg, norm, scale)
+    np.testing.assert_array_equal(ids.numpy(), want_ids)
+    np.testing.assert_allclose(w.numpy(), want_w, rtol=1e-6)
+
+
+def test_grouped_routing_with_one_group_and_no_bias_is_plain_routing():
+    gen = torch.Generator().manual_seed(21)
+    logits = torch.randn(64, 256, generator=gen)
+    ids, w, _ = moe.route_grouped(logits, None, 8, 1, 1)
+    want_ids, want_w = moe.route(logits, 8)
+    assert torch.equal(ids, want_ids)
+    torch.testing.assert_close(w, want_w, rtol=1e-6, atol=0)
+
+
+def test_grouped_routing_invariants():
+    gen = torch.Generator().manual_seed(22)
+    T, E, k, G, kg = 200, 256, 8, 8, 4
+    logits = torch.randn(T, E, generator=gen)
+    bias = 0.3 * torch.randn(E, generator=gen)
+    ids, w, choice = moe.route_grouped(logits, bias, k, G, kg, True, 2.5)
+    groups = ids // (E // G)
+    assert all(len(set(row.tolist())) <= kg for row in groups)
+    assert all(len(set(row.tolist())) == k for row in ids)
+    torch.testing.assert_close(w.sum(dim=1), torch.full((T,), 2.5), rtol=1e-5, atol=0)
+    # the bias moves the choice but not the weights: weights are ratios of unbiased sigmoids
+    score = torch.sigmoid(logits).gather(1, ids.long())
+    torch.testing.assert_close(w, 2.5 * score / score.sum(dim=1, keepdim=True), rtol=1e-5, atol=0)
+    # a large bias on one expert of a group that stays forces that expert in
+    big = bias.clone()
+    big[5] = 10.0
+    ids2, _, _ = moe.route_grouped(logits, big, k, G, kg)
+    assert (ids2[:, 0] == 5).all()
+
+
+def test_grouped_routing_matches_third_party_golden():
+    from pathlib import Path
+    z = np.load(Path(__file__).parent / 'golden' / 'router_golden.npz')
+    for tag in 'abc':
+        k, G, kg, norm = (int(v) for v in z[f'{tag}_params'])
+        logits = torch.from_numpy(z[f'{tag}_logits'])
+        # the fixture's logits are the fp32 product of its hidden states and router weight
+        want_logits = torch.from_numpy(z[f'{tag}_hidden']) @ torch.from_numpy(z[f'{tag}_weight']).T
+        torch.testing.assert_close(logits, want_logits, rtol=1e-4, atol=1e-5)
+        ids, w, _ = moe.route_grouped(logits, torch.from_numpy(z[f'{tag}_bias']), k, G, kg, bool(norm),
+                                      float(z[f'{tag}_scale'][0]))
+        order = ids.argsort(dim=-1)
+        np.testing.assert_array_equal(ids.gather(1, order).numpy(), z[f'{tag}_ids'])
+        np.testing.assert_allclose(w.gather(1, order).numpy(), z[f'{tag}_weights'], rtol=1e-5)
+
+
+def test_shared_expert_against_float64_dense():
+    x, logits, (w13_q, w13_s, w2_q, w2_s) = _tiny()
+    gen = torch.Generator().manual_seed(91)
+    (sw13_q, sw13_s, sw2_q, sw2_s) = (t[0] for t in moe.moe_make_weights(1, 256, 256, generator=gen))
+    out = moe.moe_forward_shared(x, logits, w13_q, w13_s, w2_q, w2_s, sw13_q, sw13_s, sw2_q, sw2_s, top_k=2,
+                                 out_dtype=torch.float32)
+    routed = moe.moe_forward(x, logits, w13_q, w13_s, w2_q, w2_s, top_k=2, out_dtype=torch.float32)
+    xq, xs = moe.quantize_groups(x.float())
+    xd = moe.dequantize_groups(xq, xs).double()
+    want = routed.double()
+    for t in range(x.shape[0]):
+        gu = moe.dequantize_blocks(sw13_q, sw13_s).double() @ xd[t]
+        h = gu[:256] / (1 + torch.exp(-gu[:256])) * gu[256:]
+        hq, hs = moe.quantize_groups(h.float()[None])
+        want[t] += moe.dequantize_blocks(sw2_q, sw2_s).double() @ moe.dequantize_groups(hq, hs)[0].double()
+    assert moe.rel_rms_error(out, want) < 1e-4
+    assert moe.rel_rms_error(out, routed) > 0.1       # the shared term is not negligible in this check
