@@ -184,6 +184,32 @@ def bench_conv1d(torch, capi, dev, steps, warmup, cpu_baseline):
     return res
 
 
+def bench_topk_select(torch, capi, dev, steps, warmup, cpu_baseline):
+    """The selection in front of configs[3]: 2048 of 32768 index scores per request, 64 requests."""
+    from oracle import mla
+    B, N, k = 64, 32768, 2048
+    gen = torch.Generator(device=dev).manual_seed(20259)
+    sets = [torch.randn(B, N, device=dev, generator=gen) for _ in range(8)]
+    idx = torch.empty(B, k, dtype=torch.int32, device=dev)
+    sec = timed_launches(torch, lambda i: capi.topk_select_launch(idx, sets[i % 8]), steps, warmup)
+    work = B * N * 4 + B * k * 4
+    res = dict(
+        workload="top-k selection in front of configs[3]: B=64, 2048 of 32768 fp32 index scores per request, "
+                 "seed 20259 (one workgroup per request)",
+        value=work / sec / 1e9, unit="GB/s", ms_per_step=sec * 1e3, dtype="u32", kernel="topk_select_kernel",
+        roofline=dict(bound="hbm", achieved=work / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
+                      frac=work / sec / 1e9 / HBM_PEAK_GBS, traffic=None),
+        algorithmic_bytes=work)
+    if cpu_baseline:
+        cores = len(os.sched_getaffinity(0))
+        torch.set_num_threads(cores)
+        host = sets[0].cpu()
+        csec = cpu_time(lambda: mla.topk_select(host, k))
+        res['cpu_baseline'] = dict(value=work / csec / 1e9, unit="GB/s", cores=cores, kind="port",
+                                   sample="the full selection (oracle: stable sort per request)")
+    return res
+
+
 def bench_mla(torch, capi, dev, steps, warmup, cpu_baseline, paged=False):
     from oracle import mla
     B, H, N, topk = 64, 128, 32768, 2048
@@ -329,7 +355,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=20)
     ap.add_argument('--warmup', type=int, default=5)
-    ap.add_argument('--workloads', default='gdn,gdn_fused,conv1d,moe_decode,mla,mla_paged,moe_prefill')
+    ap.add_argument('--workloads', default='gdn,gdn_fused,conv1d,moe_decode,topk_select,mla,mla_paged,moe_prefill')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run 3 plain device copies of 536 870 912 bytes (a kernel of known traffic, '
@@ -364,6 +390,8 @@ def main():
             results[name] = bench_gdn_fused(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'conv1d':
             results[name] = bench_conv1d(torch, capi, dev, args.steps, args.warmup, cpu)
+        elif name == 'topk_select':
+            results[name] = bench_topk_select(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'mla':
             results[name] = bench_mla(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'mla_paged':

@@ -31,6 +31,7 @@ SIGNATURES = {
                                                 _P]),
     'sparse_mla_decode_num_splits': (c_int, [c_int, c_int, c_int, c_int]),
     'sparse_mla_decode_workspace_bytes': (c_size_t, [c_int, c_int, c_int, c_int]),
+    'topk_select_launcher': (None, [_P, _P, _P, c_int, c_int, c_int, c_int, _P]),
     'moe_route_launcher': (None, [_P, _P, _P, c_int, c_int, c_int, c_int, _P]),
     'moe_route_grouped_launcher': (None, [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
                                           c_int, _P]),
@@ -249,6 +250,24 @@ def sparse_mla_decode_paged_launch(out, q, kv_pool, block_table, idx, workspace,
         0 if out.dtype == torch.bfloat16 else 1, config, _stream(stream))
     check_status('sparse_mla_decode_paged_launcher')
     return out
+
+
+def topk_select_launch(idx_out, scores, lengths=None, stream=None):
+    """idx_out [B, k] int32 <- indices of the k largest of scores [B, n] fp32 per row (first lengths[b]
+    entries only, if given), ties to the lower index, ascending index order, -1 padding."""
+    import torch
+    _device_contiguous(idx_out=idx_out, scores=scores)
+    B, n = scores.shape
+    _require(scores.dtype == torch.float32 and idx_out.dtype == torch.int32, 'topk_select: scores fp32, idx int32')
+    _require(idx_out.dim() == 2 and idx_out.shape[0] == B, 'topk_select: idx_out [B, k]')
+    if lengths is not None:
+        _device_contiguous(lengths=lengths)
+        _require(lengths.dtype == torch.int32 and tuple(lengths.shape) == (B,), 'topk_select: lengths int32 [B]')
+    library().topk_select_launcher(_ptr(idx_out), _ptr(scores),
+                                   _ptr(lengths) if lengths is not None else c_void_p(None), B, n,
+                                   idx_out.shape[1], 0, _stream(stream))
+    check_status('topk_select_launcher')
+    return idx_out
 
 
 MOE_WORKSPACE_FIELDS = ('ids', 'weights', 'expert_offsets', 'sorted_pairs', 'pair_pos', 'x_q', 'x_s',

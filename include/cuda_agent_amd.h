@@ -152,6 +152,16 @@ int sparse_mla_decode_num_splits(int batch, int n_heads, int topk, int config);
 /* Bytes of workspace sparse_mla_decode_launcher needs for these sizes and this config. */
 size_t sparse_mla_decode_workspace_bytes(int batch, int n_heads, int topk, int config);
 
+/* Top-k selection of index scores, the step that produces idx for the two launchers above
+ * (caller-side neighbour; same launcher pattern agent_workdir/kernels/axpby.cu:12-20):
+ *   idx_out [batch, k] int32: per request the indices of the k largest scores among the first
+ *           lengths[b] entries (all n if lengths is NULL) of scores [batch, n] fp32; ties go to
+ *           the lower index; listed in ascending index order; -1 where fewer than k candidates
+ *           exist (the attention skips them). NaN scores rank below every number.
+ * Exact (integer work on the bit patterns of the scores). config: one value (0). */
+void topk_select_launcher(int* idx_out, const float* scores, const int* lengths, int batch, int n,
+                          int k, int config, hipStream_t stream);
+
 /* ---- FP8 block-scaled MoE layer (workload configs 2 and 4 of the benchmark definition;
  * launcher pattern agent_workdir/kernels/axpby.cu:12-20). Expert weights are e4m3 with one fp32
  * scale per 128x128 block: w13_q [E, 2*inter, hidden] (rows 0..inter-1 gate, inter..2*inter-1

@@ -24,6 +24,11 @@ position p of request b -> row ``p % page_size`` of page ``block_table[b, p // p
 one pool shared by all requests. Pinned by scalar loops over divmod on small cases and by the
 identity "scatter a contiguous cache's pages into a pool under a random page permutation ->
 the paged result equals the contiguous result exactly".
+
+``topk_select`` is the selection that produces ``idx`` from index scores. Pinned by ``torch.topk`` as
+a set on tie-free rows, by scalar loops with an explicit (value, index) ordering on rows full of
+ties, signed zeros, infinities and NaNs, and by its invariants (ascending indices, every chosen
+score >= every unchosen one).
 """
 
 import math
@@ -120,6 +125,26 @@ def mla_scatter_into_pool(kv, page_size, n_spare_pages=3, generator=None):
     pool = torch.randn(n_pages, page_size, d, generator=generator).to(kv.dtype)
     pool[order] = kv.reshape(B * per_req, page_size, d).cpu()
     return pool, order.reshape(B, per_req).int()
+
+
+def topk_select(scores, k, lengths=None):
+    """Indices of the k largest scores per row among the first lengths[b] entries (all, if None):
+    ties to the lower index, ascending index order, -1 where fewer than k candidates exist; NaN ranks
+    below every number (-inf included). int32 [B, k]."""
+    B, n = scores.shape
+    out = torch.full((B, k), -1, dtype=torch.int32)
+    for b in range(B):
+        valid = n if lengths is None else max(0, min(n, int(lengths[b])))
+        row = scores[b, :valid].double()
+        nan = torch.isnan(row)
+        # stable descending sort of (is-number, value): numbers first, equal values by index
+        row = torch.where(nan, torch.full_like(row, float('-inf')), row)
+        order = torch.sort(row, descending=True, stable=True).indices
+        numbers = order[~nan[order]]
+        nans = order[nan[order]]
+        chosen = torch.cat([numbers, nans])[:k]
+        out[b, :chosen.numel()] = torch.sort(chosen).values.int()
+    return out
 
 
 def rel_rms_error(actual, expected):

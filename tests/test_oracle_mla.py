@@ -137,3 +137,48 @@ def test_unmapped_pages_drop_their_positions():
     keep[0][(idx[0] >= 8) & (idx[0] < 16)] = -1
     want = mla.sparse_mla_decode(q, kv, keep, out_dtype=torch.float32)
     assert torch.equal(mla.sparse_mla_decode_paged(q, pool, table, idx, out_dtype=torch.float32), want)
+
+
+# ---- top-k selection of index scores -----------------------------------------------------------
+
+def _select_by_loops(scores, k, lengths):
+    out = []
+    for b, row in enumerate(scores.tolist()):
+        valid = len(row) if lengths is None else max(0, min(len(row), int(lengths[b])))
+        # rank: numbers before NaN, larger first (-0 == +0), then lower index
+        ranked = sorted(range(valid), key=lambda i: (row[i] != row[i], 0.0 if row[i] != row[i] else -row[i], i))
+        chosen = sorted(ranked[:k])
+        out.append(chosen + [-1] * (k - len(chosen)))
+    return torch.tensor(out, dtype=torch.int32)
+
+
+def test_topk_select_is_torch_topk_on_tie_free_rows():
+    gen = torch.Generator().manual_seed(31)
+    scores = torch.randn(5, 300, generator=gen)
+    got = mla.topk_select(scores, 40)
+    want = torch.topk(scores, 40, dim=1).indices.sort(dim=1).values.int()
+    assert torch.equal(got, want)
+
+
+def test_topk_select_ties_specials_and_lengths():
+    gen = torch.Generator().manual_seed(32)
+    scores = torch.randint(-3, 4, (6, 50), generator=gen).float()       # many ties
+    scores[0, 5] = float('inf')
+    scores[1, 7] = float('-inf')
+    scores[2, 3::7] = float('nan')
+    scores[3, ::2] = -0.0
+    scores[3, 1::2] = 0.0
+    lengths = torch.tensor([50, 50, 50, 50, 9, 0], dtype=torch.int32)
+    for k in (1, 8, 20, 50, 64):
+        for ln in (None, lengths):
+            got = mla.topk_select(scores, k, ln)
+            assert torch.equal(got, _select_by_loops(scores, k, ln)), (k, ln)
+    # invariants on the last call: ascending, -1 padding at the end, chosen >= unchosen
+    got = mla.topk_select(scores, 8)
+    for b in range(6):
+        row = got[b]
+        assert (row[1:] > row[:-1]).all()
+        if not torch.isnan(scores[b]).any():
+            unchosen = torch.ones(50, dtype=torch.bool)
+            unchosen[row.long()] = False
+            assert scores[b, row.long()].min() >= scores[b, unchosen].max()
