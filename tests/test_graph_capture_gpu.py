@@ -97,3 +97,92 @@ def test_moe_decode_layer_in_a_graph(capi, dev):
         torch.cuda.synchronize()
         assert torch.equal(out, eager)
         eager_noise(dev)
+
+
+def test_layer_decode_chain_in_a_graph(capi, dev):
+    # convolution update -> fused GDN step, both states advancing in place across replays
+    gen = torch.Generator().manual_seed(8)
+    B, Hv, Hqk, d = 4, 8, 4, 128
+    x, cstate0, weight, bias = (t.to(dev) for t in gdn.conv_make_inputs(B, Hqk * d, Hv * d, 3, 4, torch.bfloat16,
+                                                                         generator=gen))
+    _, _, _, a, b, a_log, dt_bias, state0 = (t.to(dev) for t in gdn.gdn_make_raw_inputs(
+        B, Hv, Hqk, qkv_dtype=torch.bfloat16, generator=gen))
+
+    def buffers():
+        return dict(q=torch.empty(B, Hqk * d, dtype=torch.bfloat16, device=dev),
+                    k=torch.empty(B, Hqk * d, dtype=torch.bfloat16, device=dev),
+                    v=torch.empty(B, Hv * d, dtype=torch.bfloat16, device=dev),
+                    cstate=cstate0.clone(), state=state0.clone(), o=torch.empty(B, Hv, d, device=dev))
+
+    def step(t):
+        capi.causal_conv1d_update_launch(t['q'], t['k'], t['v'], t['cstate'], x, weight, bias)
+        capi.gdn_decode_fused_launch(t['o'], t['state'], t['q'].view(B, Hqk, d), t['k'].view(B, Hqk, d),
+                                     t['v'].view(B, Hv, d), a, b, a_log, dt_bias)
+
+    g, e = buffers(), buffers()
+    graph = capture(lambda: step(g))
+    g['cstate'].copy_(cstate0)
+    g['state'].copy_(state0)
+    for r in range(3):
+        x.copy_(torch.randn(x.shape, device=dev).bfloat16())
+        graph.replay()
+        torch.cuda.synchronize()
+        step(e)
+        torch.cuda.synchronize()
+        for name in ('q', 'k', 'v', 'cstate', 'state', 'o'):
+            assert torch.equal(g[name], e[name]), (r, name)
+        eager_noise(dev)
+
+
+def test_selection_and_paged_attention_in_a_graph(capi, dev):
+    gen = torch.Generator().manual_seed(9)
+    B, H, N, k, page = 2, 128, 1024, 256, 64
+    q, kv, _ = mla.mla_make_inputs(B, H, N, k, generator=gen)
+    pool, table = mla.mla_scatter_into_pool(kv, page, generator=gen)
+    q, pool, table = q.to(dev), pool.to(dev), table.to(dev)
+    scores = torch.randn(B, N, device=dev)
+    lengths = torch.tensor([N, 300], dtype=torch.int32, device=dev)
+    ws = torch.empty(capi.sparse_mla_workspace_bytes(B, H, k), dtype=torch.uint8, device=dev)
+
+    def step(idx, out, ws):
+        capi.topk_select_launch(idx, scores, lengths)
+        capi.sparse_mla_decode_paged_launch(out, q, pool, table, idx, ws)
+
+    idx_g, idx_e = (torch.empty(B, k, dtype=torch.int32, device=dev) for _ in range(2))
+    out_g, out_e = (torch.empty(B, H, 512, dtype=torch.bfloat16, device=dev) for _ in range(2))
+    graph = capture(lambda: step(idx_g, out_g, ws))
+    ws_e = torch.empty_like(ws)
+    for r in range(3):
+        scores.copy_(torch.randn(B, N, device=dev))
+        out_g.fill_(float('nan'))
+        graph.replay()
+        torch.cuda.synchronize()
+        step(idx_e, out_e, ws_e)
+        torch.cuda.synchronize()
+        assert torch.equal(idx_g, idx_e) and torch.equal(out_g, out_e)
+        assert torch.equal(idx_g.cpu(), mla.topk_select(scores.cpu(), k, lengths.cpu()))
+        eager_noise(dev)
+
+
+def test_moe_layer_with_shared_expert_in_a_graph(capi, dev):
+    T, H, I, E, k = 24, 512, 256, 16, 4
+    gen = torch.Generator().manual_seed(10)
+    w = [t.to(dev) for t in moe.moe_make_weights(E, H, I, gen)]
+    sw = [t[0].contiguous().to(dev) for t in moe.moe_make_weights(1, H, I, gen)]
+    x, logits = (t.to(dev) for t in moe.moe_make_inputs(T, H, E, gen))
+    ws = torch.empty(capi.moe_shared_workspace_bytes(T, H, I, I, E, k), dtype=torch.uint8, device=dev)
+    out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    graph = capture(lambda: capi.moe_fp8_shared_launch(out, x, logits, *w, *sw, ws, top_k=k))
+    eager = torch.empty_like(out)
+    ws2 = torch.empty_like(ws)
+    for r in range(3):
+        if r:
+            x.copy_(torch.randn(T, H, device=dev).bfloat16())
+            logits.copy_(torch.randn(T, E, device=dev))
+        out.fill_(float('nan'))
+        graph.replay()
+        torch.cuda.synchronize()
+        capi.moe_fp8_shared_launch(eager, x, logits, *w, *sw, ws2, top_k=k)
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
+        eager_noise(dev)
