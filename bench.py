@@ -184,6 +184,58 @@ def bench_conv1d(torch, capi, dev, steps, warmup, cpu_baseline):
     return res
 
 
+def bench_router(torch, capi, dev, steps, warmup, cpu_baseline, prefill):
+    """The router in front of configs[2] / configs[4]: logits = x . w^T in fp32, then group-limited routing with a
+    selection bias (8 groups, 4 stay, top-8)."""
+    from oracle import moe
+    T, H, E, k = (8192 if prefill else 64), 7168, 256, 8
+    gen = torch.Generator(device=dev).manual_seed(20260)
+    x = torch.randn(T, H, device=dev, generator=gen).bfloat16()
+    w = torch.randn(E, H, device=dev, generator=gen) * H ** -0.5
+    bias = 0.1 * torch.randn(E, device=dev, generator=gen)
+    logits = torch.empty(T, E, device=dev)
+    ids = torch.empty(T, k, dtype=torch.int32, device=dev)
+    wts = torch.empty(T, k, device=dev)
+    nbytes = capi.moe_router_logits_workspace_bytes(T, H, E)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev) if nbytes else None
+
+    def launch(i):
+        capi.moe_router_logits_launch(logits, x, w, ws)
+        capi.moe_route_grouped_launch(ids, wts, logits, bias, 8, 4, True, 2.5)
+
+    sec = timed_launches(torch, launch, steps, warmup)
+    flops = 2 * T * H * E
+    nbytes_alg = E * H * 4 + T * H * 2 + T * E * 4 + 2 * T * k * 4
+    if prefill:
+        res = dict(
+            workload="router in front of configs[4]: T=8192 bf16 hidden states x fp32 weight [256, 7168] -> fp32 "
+                     "logits, then group-limited biased top-8, seed 20260",
+            value=flops / sec / 1e12, unit="TFLOP/s", ms_per_step=sec * 1e3, dtype="f32",
+            kernel="moe_router_gemm_kernel",
+            roofline=dict(bound="mfma", achieved=flops / sec / 1e12, peak=157.3, unit="TFLOP/s",
+                          frac=flops / sec / 1e12 / 157.3, traffic=None),
+            algorithmic_flops=flops)
+    else:
+        res = dict(
+            workload="router in front of configs[2]: T=64 bf16 hidden states x fp32 weight [256, 7168] -> fp32 "
+                     "logits (K split 16 ways + ordered reduce), then group-limited biased top-8, seed 20260",
+            value=nbytes_alg / sec / 1e9, unit="GB/s", ms_per_step=sec * 1e3, dtype="f32",
+            kernel="moe_router_gemm_kernel",
+            roofline=dict(bound="hbm", achieved=nbytes_alg / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
+                          frac=nbytes_alg / sec / 1e9 / HBM_PEAK_GBS, traffic=None),
+            algorithmic_bytes=nbytes_alg)
+    if cpu_baseline:
+        cores = len(os.sched_getaffinity(0))
+        torch.set_num_threads(cores)
+        n_tok = min(T, 512)
+        hx, hw, hb = x[:n_tok].cpu(), w.cpu(), bias.cpu()
+        csec = cpu_time(lambda: moe.route_grouped(moe.router_logits(hx, hw), hb, 8, 8, 4, True, 2.5))
+        cval = 2 * n_tok * H * E / csec / 1e12 if prefill else nbytes_alg / csec / 1e9
+        res['cpu_baseline'] = dict(value=cval, unit=res['unit'], cores=cores, kind="port",
+                                   sample=f"tokens 0..{n_tok - 1}, eager PyTorch oracle (fp32 matmul, grouped top-k)")
+    return res
+
+
 def bench_topk_select(torch, capi, dev, steps, warmup, cpu_baseline):
     """The selection in front of configs[3]: 2048 of 32768 index scores per request, 64 requests."""
     from oracle import mla
@@ -355,7 +407,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=20)
     ap.add_argument('--warmup', type=int, default=5)
-    ap.add_argument('--workloads', default='gdn,gdn_fused,conv1d,moe_decode,topk_select,mla,mla_paged,moe_prefill')
+    ap.add_argument('--workloads', default='gdn,gdn_fused,conv1d,moe_decode,router_decode,topk_select,mla,mla_paged,moe_prefill,router_prefill')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run 3 plain device copies of 536 870 912 bytes (a kernel of known traffic, '
@@ -390,6 +442,8 @@ def main():
             results[name] = bench_gdn_fused(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'conv1d':
             results[name] = bench_conv1d(torch, capi, dev, args.steps, args.warmup, cpu)
+        elif name in ('router_decode', 'router_prefill'):
+            results[name] = bench_router(torch, capi, dev, args.steps, args.warmup, cpu, name == 'router_prefill')
         elif name == 'topk_select':
             results[name] = bench_topk_select(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'mla':

@@ -33,6 +33,9 @@ SIGNATURES = {
     'sparse_mla_decode_workspace_bytes': (c_size_t, [c_int, c_int, c_int, c_int]),
     'topk_select_launcher': (None, [_P, _P, _P, c_int, c_int, c_int, c_int, _P]),
     'moe_route_launcher': (None, [_P, _P, _P, c_int, c_int, c_int, c_int, _P]),
+    'moe_router_logits_num_splits': (c_int, [c_int, c_int, c_int]),
+    'moe_router_logits_workspace_bytes': (c_size_t, [c_int, c_int, c_int]),
+    'moe_router_logits_launcher': (None, [_P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int, c_int, _P]),
     'moe_route_grouped_launcher': (None, [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
                                           c_int, _P]),
     'moe_sort_launcher': (None, [_P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P]),
@@ -313,6 +316,30 @@ def moe_route_launch(ids, weights, logits, stream=None):
     library().moe_route_launcher(_ptr(ids), _ptr(weights), _ptr(logits), T, E, k, 0, _stream(stream))
     check_status('moe_route_launcher')
     return ids, weights
+
+
+def moe_router_logits_workspace_bytes(tokens, hidden, n_experts):
+    return int(library().moe_router_logits_workspace_bytes(tokens, hidden, n_experts))
+
+
+def moe_router_logits_launch(logits, x, w, workspace=None, stream=None):
+    """logits [T, E] fp32 <- x [T, H] (bf16 or fp32) @ w [E, H]^T (fp32); ``workspace``: uint8 device tensor of
+    ``moe_router_logits_workspace_bytes`` bytes (None when that is 0)."""
+    import torch
+    _device_contiguous(logits=logits, x=x, w=w)
+    T, H = x.shape
+    E = w.shape[0]
+    _require(x.dtype in (torch.float32, torch.bfloat16) and w.dtype == logits.dtype == torch.float32,
+             'moe_router_logits: x fp32 or bf16, w and logits fp32')
+    _require(tuple(w.shape) == (E, H) and tuple(logits.shape) == (T, E), 'moe_router_logits: shapes')
+    ws_ptr, ws_bytes = c_void_p(None), 0
+    if workspace is not None:
+        _device_contiguous(workspace=workspace)
+        ws_ptr, ws_bytes = _ptr(workspace), workspace.numel() * workspace.element_size()
+    library().moe_router_logits_launcher(_ptr(logits), _ptr(x), _ptr(w), ws_ptr, ws_bytes, T, H, E,
+                                         0 if x.dtype == torch.float32 else 1, 0, _stream(stream))
+    check_status('moe_router_logits_launcher')
+    return logits
 
 
 def moe_route_grouped_launch(ids, weights, logits, bias, n_group, topk_group, normalise=True,

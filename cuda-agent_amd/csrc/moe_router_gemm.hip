@@ -1,0 +1,195 @@
+// Router projection of a MoE layer: logits[t, e] = sum_h x[t, h] * w[e, h], fp32.
+//
+// x is the layer's bf16 (or fp32) input, w the fp32 router weight [n_experts, hidden]; both are
+// taken to fp32 exactly and multiplied on the fp32 matrix cores (v_mfma_f32_32x32x2_f32), so the
+// result differs from an fp32 reference only by the order of the additions: the routing that
+// follows compares these logits with each other, and a lower-precision product would move
+// experts across the top-k boundary.
+//
+// A wavefront owns a 32-token x 32-expert tile of the output. The MFMA pairs lane l's A value
+// (token l % 32) with lane l's B value (expert l % 32) as one k of the dot product, and any
+// assignment of k to (lane half, step) works as long as A and B agree. So for every 64 values of
+// k lane (row, half) reads the 32 consecutive values [64c + 32*half, +32) of its row: whole
+// 128-byte lines of w, 64-byte pieces of bf16 x, straight from global memory into the operand
+// registers (at 64 cycles per MFMA the loads are a small fraction of the time and need no LDS
+// staging). 4 wavefronts of a workgroup cover 64 tokens x 64 experts.
+//
+// Few tokens: K is cut into n_splits ranges (grid z) so that the weight matrix is streamed by
+// many CUs; partial sums go to a caller-provided scratch and a second kernel adds them in
+// ascending split order, so the result does not depend on timing.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "launch_status.hpp"
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int K_CHUNK = 64;
+
+// 32 consecutive values of a row as fp32
+__device__ __forceinline__ void load32(float (&dst)[32], const float* p) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const floatx4 v = reinterpret_cast<const floatx4*>(p)[i];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dst[4 * i + j] = v[j];
+    }
+}
+__device__ __forceinline__ void load32(float (&dst)[32], const uint16_t* p) {  // bf16 bits
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const u32x4 v = reinterpret_cast<const u32x4*>(p)[i];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            dst[8 * i + 2 * j] = __uint_as_float(v[j] << 16);
+            dst[8 * i + 2 * j + 1] = __uint_as_float(v[j] & 0xffff0000u);
+        }
+    }
+}
+
+// grid: x = 64-token tiles, y = 64-expert tiles, z = K split. out is logits (n_splits == 1) or
+// the partial sums [split][tokens][n_experts].
+template <typename X>
+__global__ __launch_bounds__(256) void moe_router_gemm_kernel(const X* __restrict__ x,
+                                                              const float* __restrict__ w,
+                                                              float* __restrict__ out, int tokens,
+                                                              int hidden, int n_experts,
+                                                              int chunks_per_split) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int row = lane & 31;
+    const int half = lane >> 5;
+    const int t0 = blockIdx.x * 64 + (wave & 1) * 32;
+    const int e0 = blockIdx.y * 64 + (wave >> 1) * 32;
+    if (t0 >= tokens || e0 >= n_experts) return;  // (no barrier in this kernel)
+    // rows beyond the end read the last valid row; their results are not stored
+    const int t = t0 + row < tokens ? t0 + row : tokens - 1;
+    const int e = e0 + row < n_experts ? e0 + row : n_experts - 1;
+    const int chunk_begin = blockIdx.z * chunks_per_split;
+    int chunk_end = chunk_begin + chunks_per_split;
+    const int n_chunks = hidden / K_CHUNK;
+    if (chunk_end > n_chunks) chunk_end = n_chunks;
+    const X* xp = x + (size_t)t * hidden + 32 * half;
+    const float* wp = w + (size_t)e * hidden + 32 * half;
+
+    floatx16 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    // two register sets: the loads of chunk c+1 are in flight while the MFMAs of chunk c run
+    float a0[32], b0[32], a1[32], b1[32];
+    if (chunk_begin < chunk_end) {
+        load32(a0, xp + (size_t)chunk_begin * K_CHUNK);
+        load32(b0, wp + (size_t)chunk_begin * K_CHUNK);
+    }
+    for (int c = chunk_begin; c < chunk_end; c += 2) {
+        // (past the end the last chunk is read again and not used)
+        const int c1 = c + 1 < chunk_end ? c + 1 : c;
+        load32(a1, xp + (size_t)c1 * K_CHUNK);
+        load32(b1, wp + (size_t)c1 * K_CHUNK);
+#pragma unroll
+        for (int s = 0; s < 32; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[s], b0[s], acc, 0, 0, 0);
+        if (c + 1 >= chunk_end) break;
+        const int c2 = c + 2 < chunk_end ? c + 2 : c + 1;
+        load32(a0, xp + (size_t)c2 * K_CHUNK);
+        load32(b0, wp + (size_t)c2 * K_CHUNK);
+#pragma unroll
+        for (int s = 0; s < 32; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[s], b1[s], acc, 0, 0, 0);
+    }
+    // result register i of a lane: token 8*(i/4) + 4*half + i%4 of the tile, expert `row`
+    float* dst = out + (size_t)blockIdx.z * tokens * n_experts;
+    if (e0 + row < n_experts) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int tt = t0 + 8 * (i / 4) + 4 * half + (i % 4);
+            if (tt < tokens) dst[(size_t)tt * n_experts + e0 + row] = acc[i];
+        }
+    }
+}
+
+// logits = partial[0] + partial[1] + ... in that order
+__global__ __launch_bounds__(256) void moe_router_reduce_kernel(const float* __restrict__ partial,
+                                                                float* __restrict__ logits,
+                                                                size_t count, int n_splits) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= count) return;
+    // eight loads at a time are in flight; the additions stay in ascending split order
+    float sum = 0.f;
+    for (int s0 = 0; s0 < n_splits; s0 += 8) {
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = s0 + j < n_splits ? partial[(size_t)(s0 + j) * count + i] : 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            if (s0 + j < n_splits) sum = (s0 + j == 0) ? v[j] : sum + v[j];
+    }
+    logits[i] = sum;
+}
+
+int pick_router_splits(int tokens, int hidden, int n_experts) {
+    const long tiles = (long)((tokens + 63) / 64) * ((n_experts + 63) / 64);
+    const int n_chunks = hidden / K_CHUNK;
+    int splits = 1;
+    // aim at about two workgroups per CU; every split keeps at least 2 chunks
+    while (tiles * splits < 512 && splits * 2 * 2 <= n_chunks) splits *= 2;
+    return splits;
+}
+
+}  // namespace
+
+// K splits the launcher uses for these sizes (1 = no scratch needed)
+extern "C" int moe_router_logits_num_splits(int tokens, int hidden, int n_experts) {
+    if (tokens <= 0 || hidden <= 0 || n_experts <= 0 || hidden % K_CHUNK != 0) return 0;
+    return pick_router_splits(tokens, hidden, n_experts);
+}
+
+// bytes of scratch moe_router_logits_launcher needs (0 when K is not split)
+extern "C" size_t moe_router_logits_workspace_bytes(int tokens, int hidden, int n_experts) {
+    const int splits = moe_router_logits_num_splits(tokens, hidden, n_experts);
+    return splits <= 1 ? 0 : (size_t)splits * tokens * n_experts * sizeof(float);
+}
+
+// logits [tokens, n_experts] fp32 = x [tokens, hidden] (x_dtype 0 = fp32, 1 = bf16) times
+// w [n_experts, hidden] fp32, transposed. hidden a multiple of 64; x and w 16-byte aligned.
+// workspace: moe_router_logits_workspace_bytes(...) bytes of device scratch (may be null if 0).
+extern "C" void moe_router_logits_launcher(float* logits, const void* x, const float* w,
+                                           void* workspace, size_t workspace_bytes, int tokens,
+                                           int hidden, int n_experts, int x_dtype, int config,
+                                           hipStream_t stream) {
+    (void)config;
+    if (tokens <= 0 || n_experts <= 0) return;
+    if (hidden <= 0 || hidden % K_CHUNK != 0 || (x_dtype != 0 && x_dtype != 1) ||
+        (tokens + 63) / 64 > 0x7fffffff / 64 || (n_experts + 63) / 64 > 65535) {
+        caa::set_status(CAA_UNSUPPORTED_SHAPE);
+        return;
+    }
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w) |
+                           reinterpret_cast<uintptr_t>(workspace);
+    if (!logits || !x || !w || (bits & 15u) != 0) {
+        caa::set_status(CAA_BAD_ARGUMENT);
+        return;
+    }
+    const int splits = pick_router_splits(tokens, hidden, n_experts);
+    const size_t need = splits <= 1 ? 0 : (size_t)splits * tokens * n_experts * sizeof(float);
+    if (need > 0 && (!workspace || workspace_bytes < need)) {
+        caa::set_status(CAA_WORKSPACE_TOO_SMALL);
+        return;
+    }
+    const int n_chunks = hidden / K_CHUNK;
+    const int chunks_per_split = (n_chunks + splits - 1) / splits;
+    float* out = splits > 1 ? static_cast<float*>(workspace) : logits;
+    const dim3 grid((tokens + 63) / 64, (n_experts + 63) / 64, splits);
+    if (x_dtype == 0) {
+        moe_router_gemm_kernel<float><<<grid, 256, 0, stream>>>(
+            static_cast<const float*>(x), w, out, tokens, hidden, n_experts, chunks_per_split);
+    } else {
+        moe_router_gemm_kernel<uint16_t><<<grid, 256, 0, stream>>>(
+            static_cast<const uint16_t*>(x), w, out, tokens, hidden, n_experts, chunks_per_split);
+    }
+    if (splits > 1) {
+        const size_t count = (size_t)tokens * n_experts;
+        moe_router_reduce_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>(
+            static_cast<const float*>(workspace), logits, count, splits);
+    }
+}

@@ -177,6 +177,19 @@ void topk_select_launcher(int* idx_out, const float* scores, const int* lengths,
 void moe_route_launcher(int* ids, float* weights, const float* logits, int tokens, int n_experts,
                         int top_k, int config, hipStream_t stream);
 
+/* Router projection in front of the routing (caller-side neighbour, same launcher pattern):
+ *   logits [tokens, n_experts] fp32 = x [tokens, hidden] . w [n_experts, hidden]^T
+ * x fp32 (x_dtype 0) or bf16 (1), w fp32; both enter the fp32 matrix cores exactly, so the result
+ * differs from an fp32 reference only by the order of the additions. hidden a multiple of 64;
+ * x, w and workspace 16-byte aligned. For few tokens K is split over workgroups and the partial
+ * sums are added in a fixed order from workspace: moe_router_logits_workspace_bytes(...) bytes
+ * (0, and workspace may be NULL, when moe_router_logits_num_splits(...) is 1). */
+int moe_router_logits_num_splits(int tokens, int hidden, int n_experts);
+size_t moe_router_logits_workspace_bytes(int tokens, int hidden, int n_experts);
+void moe_router_logits_launcher(float* logits, const void* x, const float* w, void* workspace,
+                                size_t workspace_bytes, int tokens, int hidden, int n_experts,
+                                int x_dtype, int config, hipStream_t stream);
+
 /* Group-limited routing with a selection bias, the router of DeepSeek-V3-style layers (caller-
  * side neighbour of moe_route_launcher; same launcher pattern):
  *   score = sigmoid(logit), choice = score + bias; a group (n_experts/n_group consecutive

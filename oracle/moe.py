@@ -26,7 +26,8 @@ choice with a selection bias; no counterpart in the reference repository). Pinne
 on small sizes, by the reduction to ``route`` when there is one group and no bias, by its
 invariants (chosen experts lie in exactly topk_group groups, weights sum to the scaling factor),
 and by a golden fixture written from the third-party ``transformers`` router
-(tests/golden/make_router_golden.py).
+(tests/golden/make_router_golden.py). ``router_logits`` is the projection in front of it, pinned by a float64
+product and by the same fixture's logits.
 
 ``moe_forward_shared`` adds the shared expert of such a layer; it is built from ``moe_forward`` itself
 and pinned by a float64 dense evaluation of the same sum on a tiny shape.
@@ -120,6 +121,12 @@ def route(logits, top_k=8):
     order = torch.sort(logits, dim=-1, descending=True, stable=True).indices[:, :top_k]
     score = torch.sigmoid(logits.float()).gather(1, order)
     return order.int(), score / score.sum(dim=-1, keepdim=True)
+
+
+def router_logits(x, w):
+    """logits [T,E] fp32 = x [T,H] (bf16 or fp32, taken to fp32) @ w [E,H]^T (fp32), as the third-party
+    router computes them (``F.linear`` of the two fp32 casts)."""
+    return x.float() @ w.float().T
 
 
 def route_grouped(logits, bias, top_k, n_group, topk_group, normalise=True, routed_scaling_factor=1.0):

@@ -110,3 +110,79 @@ def test_rejects_unsupported_shapes(capi, dev):
     with pytest.raises(capi.LaunchRejected):
         capi.moe_route_grouped_launch(ids, w, logits, None, 8, 1)
     torch.cuda.synchronize()
+
+
+# ---- router projection ---------------------------------------------------------------------------
+
+def run_logits(capi, dev, x, w):
+    T, H = x.shape
+    E = w.shape[0]
+    logits = torch.full((T, E), float('nan'), device=dev)
+    nbytes = capi.moe_router_logits_workspace_bytes(T, H, E)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev) if nbytes else None
+    capi.moe_router_logits_launch(logits, x.to(dev), w.to(dev), ws)
+    torch.cuda.synchronize()
+    return logits.cpu()
+
+
+def logits_bound(x, w):
+    # fp32 accumulation of H products in any order: |err| <= H * 2^-24 * sum |x_h w_eh| (loose by sqrt(H))
+    return x.shape[1] * 2.0 ** -24 * (x.double().abs() @ w.double().abs().T)
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('shape', [(64, 7168, 256), (1, 64, 32), (100, 448, 72), (700, 1024, 256), (33, 128, 1),
+                                   (130, 2048, 384)])
+def test_router_logits_match_float64(capi, dev, shape, dtype):
+    T, H, E = shape
+    gen = torch.Generator().manual_seed(T + E)
+    x = torch.randn(T, H, generator=gen).to(dtype)
+    w = torch.randn(E, H, generator=gen) * H ** -0.5
+    got = run_logits(capi, dev, x, w)
+    want = x.double() @ w.double().T
+    assert torch.isfinite(got).all()
+    assert ((got.double() - want).abs() <= logits_bound(x, w)).all()
+    # as close to the exact product as the oracle's own fp32 evaluation
+    err = (got.double() - want).abs().max().item()
+    ref_err = (moe.router_logits(x, w).double() - want).abs().max().item()
+    assert err <= 4 * ref_err + 1e-7
+
+
+def test_router_logits_exact_on_integers(capi, dev):
+    # small integers: every partial sum is an exact fp32 integer, so any summation order gives the same bits
+    gen = torch.Generator().manual_seed(51)
+    x = torch.randint(-8, 9, (96, 512), generator=gen).float().bfloat16()
+    w = torch.randint(-8, 9, (64, 512), generator=gen).float()
+    assert torch.equal(run_logits(capi, dev, x, w), x.float() @ w.T)
+
+
+def test_router_logits_golden_fixture(capi, dev):
+    z = np.load(Path(__file__).parent / 'golden' / 'router_golden.npz')
+    for tag in 'a':                       # (the other two cases have hidden = 32, below the kernel's 64 grain)
+        got = run_logits(capi, dev, torch.from_numpy(z[f'{tag}_hidden']).bfloat16(), torch.from_numpy(z[f'{tag}_weight']))
+        torch.testing.assert_close(got, torch.from_numpy(z[f'{tag}_logits']), rtol=1e-5, atol=1e-6)
+
+
+def test_projection_then_grouped_routing_at_prefill_size(capi, dev):
+    # hidden states -> logits -> experts, against the oracle's chain; a token may differ only on a near-tie
+    gen = torch.Generator().manual_seed(52)
+    T, H, E = 8192, 1024, 256
+    x = torch.randn(T, H, generator=gen).bfloat16()
+    w = torch.randn(E, H, generator=gen) * H ** -0.5
+    bias = 0.1 * torch.randn(E, generator=gen)
+    logits = run_logits(capi, dev, x, w)
+    ids, _ = run_kernel(capi, dev, logits, bias, 8, 8, 4, True, 2.5)
+    want_ids, _, _ = moe.route_grouped(moe.router_logits(x, w), bias, 8, 8, 4, True, 2.5)
+    differing = (ids != want_ids).any(dim=1).sum().item()
+    assert differing <= 8, differing        # logits differ in the last place: 1 token in 1000 may flip
+
+
+def test_router_logits_rejects_bad_arguments(capi, dev):
+    logits = torch.zeros(4, 32, device=dev)
+    w = torch.zeros(32, 96, device=dev)
+    with pytest.raises(capi.LaunchRejected):          # hidden not a multiple of 64
+        capi.moe_router_logits_launch(logits, torch.zeros(4, 96, device=dev), w)
+    w = torch.zeros(32, 7168, device=dev)
+    with pytest.raises(capi.LaunchRejected):          # K is split for 4 tokens: scratch needed
+        capi.moe_router_logits_launch(logits, torch.zeros(4, 7168, device=dev), w)
+    torch.cuda.synchronize()

@@ -273,3 +273,18 @@ def test_shared_expert_against_float64_dense():
         want[t] += moe.dequantize_blocks(sw2_q, sw2_s).double() @ moe.dequantize_groups(hq, hs)[0].double()
     assert moe.rel_rms_error(out, want) < 1e-4
     assert moe.rel_rms_error(out, routed) > 0.1       # the shared term is not negligible in this check
+
+
+def test_router_logits_against_float64_and_golden():
+    from pathlib import Path
+    gen = torch.Generator().manual_seed(23)
+    x = torch.randn(20, 192, generator=gen).bfloat16()
+    w = torch.randn(48, 192, generator=gen)
+    got = moe.router_logits(x, w)
+    want = x.double() @ w.double().T
+    assert got.dtype == torch.float32
+    torch.testing.assert_close(got.double(), want, rtol=1e-5, atol=1e-5)
+    z = np.load(Path(__file__).parent / 'golden' / 'router_golden.npz')
+    for tag in 'abc':
+        got = moe.router_logits(torch.from_numpy(z[f'{tag}_hidden']).bfloat16(), torch.from_numpy(z[f'{tag}_weight']))
+        torch.testing.assert_close(got, torch.from_numpy(z[f'{tag}_logits']), rtol=1e-5, atol=1e-6)
