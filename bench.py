@@ -388,6 +388,17 @@ def bench_moe(torch, capi, dev, steps, warmup, cpu_baseline, prefill):
         value=flops2 / sec2 / 1e12 if prefill else wbytes2 / sec2 / 1e9,
         note="moe_fp8_shared_launcher: the layer above plus one shared expert of inter 2048, seed 20258")
     del ws2
+    # the same layer with power-of-two (UE8M0) block scales: the weight scales rounded up to powers of two,
+    # activations quantised with power-of-two scales, the tiled GEMMs scaled by the MFMA itself
+    p13_s = torch.exp2(torch.ceil(torch.log2(w13_s)))
+    p2_s = torch.exp2(torch.ceil(torch.log2(w2_s)))
+    ws3 = torch.empty(capi.moe_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device=dev)
+    sec3 = timed_launches(
+        torch, lambda i: capi.moe_fp8_launch(out, x, logits, w13_q, p13_s, w2_q, p2_s, ws3, config=32), steps, warmup)
+    res['with_ue8m0_scales'] = dict(
+        ms_per_step=sec3 * 1e3, unit=res['unit'], value=flops / sec3 / 1e12 if prefill else wbytes / sec3 / 1e9,
+        note="moe_fp8_launcher with config 32: the same workload with every block scale a power of two")
+    del ws3
     if cpu_baseline:
         n_tok = 4
         csec, n_used, cores = moe_cpu_baseline(torch, tensors, n_tok)

@@ -380,14 +380,17 @@ def moe_sort_launch(ids, n_experts, stream=None):
     return sorted_pairs, pair_pos, offsets
 
 
-def moe_quant_bf16_launch(q, scales, x, stream=None):
+CONFIG_UE8M0 = 32   # config bit of the MoE launchers: power-of-two block scales
+
+
+def moe_quant_bf16_launch(q, scales, x, stream=None, config=0):
     import torch
     _device_contiguous(q=q, scales=scales, x=x)
     R, C = x.shape
     _require(x.dtype == torch.bfloat16 and scales.dtype == torch.float32, 'moe_quant: dtypes')
     _require(q.element_size() == 1 and tuple(q.shape) == (R, C), 'moe_quant: q must be 1-byte [R, C]')
     _require(tuple(scales.shape) == (R, C // 128), 'moe_quant: scales shape')
-    library().moe_quant_bf16_launcher(_ptr(q), _ptr(scales), _ptr(x), R, C, 0, _stream(stream))
+    library().moe_quant_bf16_launcher(_ptr(q), _ptr(scales), _ptr(x), R, C, config, _stream(stream))
     check_status('moe_quant_bf16_launcher')
     return q, scales
 

@@ -13,6 +13,24 @@ constexpr float INV_E4M3_MAX = (float)(1.0 / 448.0);  // scales are amax times t
 constexpr float AMAX_FLOOR = 1e-12f;  // an all-zero group gets the scale 1e-12 * fp32(1/448)
 constexpr int SORT_CHUNK_TOKENS = 256;
 
+// config bit of the layer, quantiser and gate/up launchers: block scales are powers of two (the UE8M0
+// convention: 8 exponent bits, no mantissa). The caller's weight scales must then be powers of two; the
+// activation scales become the smallest power of two >= amax / 448.
+constexpr int CONFIG_UE8M0 = 32;
+
+#ifdef __HIPCC__
+// scale of a 128-wide activation group with maximum magnitude amax
+__device__ __forceinline__ float group_scale(float amax, bool pow2) {
+    amax = fmaxf(amax, AMAX_FLOOR);
+    if (!pow2) return amax * INV_E4M3_MAX;
+    // amax = (1 + m) * 2^k and 448 = 1.75 * 2^8: the smallest power of two that is >= amax / 448 is
+    // 2^(k-8) if m <= 0.75, else 2^(k-7). Exact: integer work on the bit pattern.
+    const uint32_t u = __float_as_uint(amax);
+    const uint32_t exponent = (u >> 23) - 8u + ((u & 0x7fffffu) > 0x600000u ? 1u : 0u);
+    return __uint_as_float(exponent << 23);
+}
+#endif
+
 // Device scratch of one forward pass, carved from the caller's workspace.
 struct Workspace {
     int* ids;             // [T*k]  expert of every (token, slot) pair, slots by descending logit

@@ -45,7 +45,7 @@ __global__ __launch_bounds__(256) void moe_stream_gemm_kernel(
     const uint8_t* __restrict__ w_q, const float* __restrict__ w_s, const uint8_t* __restrict__ a_q,
     const float* __restrict__ a_s, const int* __restrict__ sorted_pairs,
     const int* __restrict__ expert_offsets, uint8_t* __restrict__ h_q, float* __restrict__ h_s,
-    float* __restrict__ y, int K, int n_rows, int inter, int top_k) {
+    float* __restrict__ y, int K, int n_rows, int inter, int top_k, bool pow2) {
     constexpr int TILES = GATE_UP ? 4 : 2;
     __shared__ float s_amax[4][NT * 16];
 
@@ -163,7 +163,7 @@ __global__ __launch_bounds__(256) void moe_stream_gemm_kernel(
                 const int idx = nt * 16 + col;
                 const float amax =
                     fmaxf(fmaxf(s_amax[0][idx], s_amax[1][idx]), fmaxf(s_amax[2][idx], s_amax[3][idx]));
-                const float scale = fmaxf(amax, AMAX_FLOOR) * INV_E4M3_MAX;
+                const float scale = group_scale(amax, pow2);
                 if (pos[nt] < end) {
 #pragma unroll
                     for (int i = 0; i < 2; ++i) {
@@ -243,7 +243,7 @@ __global__ __launch_bounds__(256) void moe_stream_gemm_lds_kernel(
     const uint8_t* __restrict__ w_q, const float* __restrict__ w_s, const uint8_t* __restrict__ a_q,
     const float* __restrict__ a_s, const int* __restrict__ sorted_pairs,
     const int* __restrict__ expert_offsets, uint8_t* __restrict__ h_q, float* __restrict__ h_s,
-    float* __restrict__ y, int K, int n_rows, int inter, int top_k) {
+    float* __restrict__ y, int K, int n_rows, int inter, int top_k, bool pow2) {
     constexpr int TILES = 4;
     constexpr int DEPTH = 3;
     constexpr int TILE_BYTES = 16 * GROUP;                       // 2 KB
@@ -413,7 +413,7 @@ __global__ __launch_bounds__(256) void moe_stream_gemm_lds_kernel(
                 const int idx = nt * 16 + col;
                 const float amax =
                     fmaxf(fmaxf(s_amax[0][idx], s_amax[1][idx]), fmaxf(s_amax[2][idx], s_amax[3][idx]));
-                const float scale = fmaxf(amax, AMAX_FLOOR) * INV_E4M3_MAX;
+                const float scale = group_scale(amax, pow2);
                 if (pos[nt] < end) {
 #pragma unroll
                     for (int i = 0; i < 2; ++i) {
@@ -476,6 +476,8 @@ extern "C" void moe_gate_up_launcher(void* h_q, float* h_s, const void* x_q, con
     auto* hq = static_cast<uint8_t*>(h_q);
     const auto* xq = static_cast<const uint8_t*>(x_q);
     const auto* wq = static_cast<const uint8_t*>(w13_q);
+    const bool pow2 = (config & CONFIG_UE8M0) != 0;
+    config &= ~CONFIG_UE8M0;
     int nt = config & 7;
     if (nt != 1 && nt != 2 && nt != 4) {
         const long avg = (long)tokens * top_k / n_experts;  // pairs per expert if spread evenly
@@ -487,28 +489,28 @@ extern "C" void moe_gate_up_launcher(void* h_q, float* h_s, const void* x_q, con
             if (lds_path) {
                 moe_stream_gemm_lds_kernel<true, 1><<<grid, 256, 0, stream>>>(
                     wq, w13_s, xq, x_s, sorted_pairs, expert_offsets, hq, h_s, nullptr, hidden,
-                    2 * inter, inter, top_k);
+                    2 * inter, inter, top_k, pow2);
             } else {
                 moe_stream_gemm_kernel<true, 1><<<grid, 256, 0, stream>>>(
                     wq, w13_s, xq, x_s, sorted_pairs, expert_offsets, hq, h_s, nullptr, hidden,
-                    2 * inter, inter, top_k);
+                    2 * inter, inter, top_k, pow2);
             }
             break;
         case 2:
             if (lds_path) {
                 moe_stream_gemm_lds_kernel<true, 2><<<grid, 256, 0, stream>>>(
                     wq, w13_s, xq, x_s, sorted_pairs, expert_offsets, hq, h_s, nullptr, hidden,
-                    2 * inter, inter, top_k);
+                    2 * inter, inter, top_k, pow2);
             } else {
                 moe_stream_gemm_kernel<true, 2><<<grid, 256, 0, stream>>>(
                     wq, w13_s, xq, x_s, sorted_pairs, expert_offsets, hq, h_s, nullptr, hidden,
-                    2 * inter, inter, top_k);
+                    2 * inter, inter, top_k, pow2);
             }
             break;
         default:
             moe_stream_gemm_kernel<true, 4><<<grid, 256, 0, stream>>>(
                 wq, w13_s, xq, x_s, sorted_pairs, expert_offsets, hq, h_s, nullptr, hidden, 2 * inter,
-                inter, top_k);
+                inter, top_k, pow2);
             break;
     }
 }
@@ -533,6 +535,7 @@ extern "C" void moe_down_launcher(float* y, const void* h_q, const float* h_s, c
     const dim3 grid(hidden / GROUP, n_experts);
     const auto* hq = static_cast<const uint8_t*>(h_q);
     const auto* wq = static_cast<const uint8_t*>(w2_q);
+    config &= ~CONFIG_UE8M0;  // (the down GEMM has no requantisation: nothing depends on the scale convention)
     int nt = config & 7;
     if (nt != 1 && nt != 2 && nt != 4) {
         const long avg = (long)tokens * top_k / n_experts;
@@ -545,28 +548,28 @@ extern "C" void moe_down_launcher(float* y, const void* h_q, const float* h_s, c
             if (lds_path) {
                 moe_stream_gemm_lds_kernel<false, 1><<<grid256, 256, 0, stream>>>(
                     wq, w2_s, hq, h_s, nullptr, expert_offsets, nullptr, nullptr, y, inter, hidden,
-                    inter, top_k);
+                    inter, top_k, false);
             } else {
                 moe_stream_gemm_kernel<false, 1><<<grid, 256, 0, stream>>>(
                     wq, w2_s, hq, h_s, nullptr, expert_offsets, nullptr, nullptr, y, inter, hidden,
-                    inter, top_k);
+                    inter, top_k, false);
             }
             break;
         case 2:
             if (lds_path) {
                 moe_stream_gemm_lds_kernel<false, 2><<<grid256, 256, 0, stream>>>(
                     wq, w2_s, hq, h_s, nullptr, expert_offsets, nullptr, nullptr, y, inter, hidden,
-                    inter, top_k);
+                    inter, top_k, false);
             } else {
                 moe_stream_gemm_kernel<false, 2><<<grid, 256, 0, stream>>>(
                     wq, w2_s, hq, h_s, nullptr, expert_offsets, nullptr, nullptr, y, inter, hidden,
-                    inter, top_k);
+                    inter, top_k, false);
             }
             break;
         default:
             moe_stream_gemm_kernel<false, 4><<<grid, 256, 0, stream>>>(
                 wq, w2_s, hq, h_s, nullptr, expert_offsets, nullptr, nullptr, y, inter, hidden, inter,
-                top_k);
+                top_k, false);
             break;
     }
 }

@@ -12,7 +12,8 @@
 //   the unscaled partial of one 128-block (two MFMAs of K = 64) is folded into the fp32
 //   accumulator with one multiply-add per value (the block scales are arbitrary fp32 and vary
 //   along K, so they can be applied neither once at the end nor by the hardware's
-//   power-of-two block scaling);
+//   power-of-two block scaling; when the caller declares them powers of two, the UE8M0 form
+//   of the kernel hands them to the MFMA instead);
 //   the two A tiles of a wavefront stay in registers for the whole block while the four B
 //   tiles stream through: 24 KB of LDS reads per wavefront and block, 16 MFMAs.
 //
@@ -142,7 +143,11 @@ __device__ unsigned long long g_phase_cycles[8][8];
 #endif
 
 // grid: 1-D, see the mapping at the top of the kernel
-template <bool GATE_UP>
+// UE8M0: all block scales are powers of two. They then go into the MFMA as its per-operand block scale
+// (v_mfma_scale_f32_32x32x64_f8f6f4: each lane's 32 values of A and of B are multiplied by
+// 2^(byte - 127)), the products of all K blocks add up in the accumulator itself, and the per-block
+// multiply-add on the VALU (128 per wavefront and K block) disappears.
+template <bool GATE_UP, bool UE8M0>
 __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
     const uint8_t* __restrict__ w_q, const float* __restrict__ w_s, const uint8_t* __restrict__ a_q,
     const float* __restrict__ as_t, const int* __restrict__ sorted_pairs,
@@ -318,6 +323,28 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
         }
         const float w0 = ws0[kb];
         const float w1 = ws1[kb];
+        if constexpr (UE8M0) {
+            // exponent bytes of the three scales; opsel 0 = byte 0 of the scale register
+            const int e0 = (int)((__float_as_uint(w0) >> 23) & 255u);
+            const int e1 = (int)((__float_as_uint(w1) >> 23) & 255u);
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const int eb = (int)((__float_as_uint(bs) >> 23) & 255u);
+                acc[0][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(A[0][0], B[0], acc[0][b], 0, 0, 0, e0, 0, eb);
+                acc[1][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(A[1][0], B[0], acc[1][b], 0, 0, 0, e1, 0, eb);
+                loads(2 * b);
+                __builtin_amdgcn_sched_barrier(0);
+                acc[0][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(A[0][1], B[1], acc[0][b], 0, 0, 0, e0, 0, eb);
+                acc[1][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(A[1][1], B[1], acc[1][b], 0, 0, 0, e1, 0, eb);
+                if (b + 1 < NB) {
+                    read_b(b + 1);
+                    bs = read_bs(b + 1);
+                }
+                loads(2 * b + 1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            return;
+        }
         floatx16 p0, p1;
         float s1_prev = 0.f;
 #pragma unroll
@@ -414,7 +441,7 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
             const int pl = th * 128 + b * 32 + r32;
             const float m = fmaxf(fmaxf(s_amax[pl], s_amax[TILE_PAIRS + pl]),
                                   fmaxf(s_amax[2 * TILE_PAIRS + pl], s_amax[3 * TILE_PAIRS + pl]));
-            const float scale = fmaxf(m, AMAX_FLOOR) * INV_E4M3_MAX;
+            const float scale = group_scale(m, UE8M0);
 #pragma unroll
             for (int qd = 0; qd < 4; ++qd) {
                 float q[4];
@@ -502,7 +529,7 @@ extern "C" void moe_gate_up_tiled_launcher(void* h_q, float* h_s, float* hs_t, c
                                            const float* xs_t, const void* w13_q, const float* w13_s,
                                            const int* sorted_pairs, const int* expert_offsets,
                                            const int* tile_start, int tokens, int hidden, int inter,
-                                           int n_experts, int top_k, int scale_stride,
+                                           int n_experts, int top_k, int scale_stride, int ue8m0,
                                            hipStream_t stream) {
     if (tokens <= 0) return;
     if (hidden % GROUP != 0 || inter % GROUP != 0 || hidden <= 0 || inter <= 0 ||
@@ -512,7 +539,8 @@ extern "C" void moe_gate_up_tiled_launcher(void* h_q, float* h_s, float* hs_t, c
     }
     const int max_tiles = (tokens * top_k) / TILE_PAIRS + n_experts;
     const dim3 grid(tiled_grid(inter / GROUP, max_tiles));
-    moe_tiled_gemm_kernel<true><<<grid, 512, 0, stream>>>(
+    const auto kernel = ue8m0 ? moe_tiled_gemm_kernel<true, true> : moe_tiled_gemm_kernel<true, false>;
+    kernel<<<grid, 512, 0, stream>>>(
         static_cast<const uint8_t*>(w13_q), w13_s, static_cast<const uint8_t*>(x_q), xs_t, sorted_pairs,
         expert_offsets, tile_start, static_cast<uint8_t*>(h_q), h_s, hs_t, nullptr, hidden, 2 * inter,
         inter, top_k, n_experts, scale_stride);
@@ -521,7 +549,8 @@ extern "C" void moe_gate_up_tiled_launcher(void* h_q, float* h_s, float* hs_t, c
 extern "C" void moe_down_tiled_launcher(float* y, const void* h_q, const float* hs_t, const void* w2_q,
                                         const float* w2_s, const int* expert_offsets,
                                         const int* tile_start, int tokens, int hidden, int inter,
-                                        int n_experts, int top_k, int scale_stride, hipStream_t stream) {
+                                        int n_experts, int top_k, int scale_stride, int ue8m0,
+                                        hipStream_t stream) {
     if (tokens <= 0) return;
     if (hidden % TILE_ROWS != 0 || inter % GROUP != 0 || hidden <= 0 || inter <= 0 ||
         (unsigned long long)tokens * top_k * inter >= (1ull << 32)) {  // 32-bit activation offsets
@@ -530,7 +559,8 @@ extern "C" void moe_down_tiled_launcher(float* y, const void* h_q, const float* 
     }
     const int max_tiles = (tokens * top_k) / TILE_PAIRS + n_experts;
     const dim3 grid(tiled_grid(hidden / TILE_ROWS, max_tiles));
-    moe_tiled_gemm_kernel<false><<<grid, 512, 0, stream>>>(
+    const auto kernel = ue8m0 ? moe_tiled_gemm_kernel<false, true> : moe_tiled_gemm_kernel<false, false>;
+    kernel<<<grid, 512, 0, stream>>>(
         static_cast<const uint8_t*>(w2_q), w2_s, static_cast<const uint8_t*>(h_q), hs_t, nullptr,
         expert_offsets, tile_start, nullptr, nullptr, nullptr, y, inter, hidden, inter, top_k,
         n_experts, scale_stride);

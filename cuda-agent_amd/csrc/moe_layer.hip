@@ -32,12 +32,13 @@ extern "C" void moe_gate_up_tiled_launcher(void* h_q, float* h_s, float* hs_t, c
                                            const float* xs_t, const void* w13_q, const float* w13_s,
                                            const int* sorted_pairs, const int* expert_offsets,
                                            const int* tile_start, int tokens, int hidden, int inter,
-                                           int n_experts, int top_k, int scale_stride,
+                                           int n_experts, int top_k, int scale_stride, int ue8m0,
                                            hipStream_t stream);
 extern "C" void moe_down_tiled_launcher(float* y, const void* h_q, const float* hs_t, const void* w2_q,
                                         const float* w2_s, const int* expert_offsets,
                                         const int* tile_start, int tokens, int hidden, int inter,
-                                        int n_experts, int top_k, int scale_stride, hipStream_t stream);
+                                        int n_experts, int top_k, int scale_stride, int ue8m0,
+                                        hipStream_t stream);
 
 namespace {
 
@@ -162,6 +163,8 @@ namespace {
 void run_expert_gemms(const moe::Workspace& w, const void* w13_q, const float* w13_s,
                       const void* w2_q, const float* w2_s, int tokens, int hidden, int inter,
                       int n_experts, int top_k, int config, hipStream_t stream) {
+    const int ue8m0 = config & CONFIG_UE8M0;  // power-of-two block scales, see moe_fp8_launcher
+    config &= ~CONFIG_UE8M0;
     // (the tiled kernels address activations with 32-bit byte offsets)
     const bool fits32 = (unsigned long long)tokens * hidden < (1ull << 32) &&
                         (unsigned long long)tokens * top_k * inter < (1ull << 32);
@@ -172,12 +175,12 @@ void run_expert_gemms(const moe::Workspace& w, const void* w13_q, const float* w
                                    hidden, n_experts, top_k, w.scale_stride, stream);
         moe_gate_up_tiled_launcher(w.h_q, w.h_s, w.hs_t, w.x_q, w.xs_t, w13_q, w13_s, w.sorted_pairs,
                                    w.expert_offsets, w.tile_start, tokens, hidden, inter, n_experts,
-                                   top_k, w.scale_stride, stream);
+                                   top_k, w.scale_stride, ue8m0, stream);
         moe_down_tiled_launcher(w.y, w.h_q, w.hs_t, w2_q, w2_s, w.expert_offsets, w.tile_start, tokens,
-                                hidden, inter, n_experts, top_k, w.scale_stride, stream);
+                                hidden, inter, n_experts, top_k, w.scale_stride, ue8m0, stream);
     } else {
         moe_gate_up_launcher(w.h_q, w.h_s, w.x_q, w.x_s, w13_q, w13_s, w.sorted_pairs, w.expert_offsets,
-                             tokens, hidden, inter, n_experts, top_k, config, stream);
+                             tokens, hidden, inter, n_experts, top_k, config | ue8m0, stream);
         moe_down_launcher(w.y, w.h_q, w.h_s, w2_q, w2_s, w.expert_offsets, tokens, hidden, inter,
                           n_experts, top_k, config, stream);
     }
@@ -194,6 +197,9 @@ bool layer_shape_ok(int hidden, int inter, int n_experts, int top_k, int tokens,
 // The whole layer. out [tokens, hidden] bf16 (out_dtype 0) or fp32 (out_dtype 1).
 // config: 0 = choose by the average number of pairs per expert (above 32: LDS-tiled GEMMs, else
 // weight streaming); 16 forces the tiled GEMMs; 1, 2, 4 (+8) force streaming, see moe_gate_up_launcher.
+// +32: all block scales are powers of two (UE8M0). The caller's weight scales must be; x and h are
+// then quantised with the smallest power-of-two scale >= amax/448, and the tiled GEMMs let the MFMA
+// apply the scales (no per-block multiply-add on the VALU).
 extern "C" void moe_fp8_launcher(void* out, const void* x, const float* logits, const void* w13_q,
                                  const float* w13_s, const void* w2_q, const float* w2_s,
                                  void* workspace, size_t workspace_bytes, int tokens, int hidden,
@@ -216,7 +222,7 @@ extern "C" void moe_fp8_launcher(void* out, const void* x, const float* logits, 
     }
     moe_route_sort_launcher(w.ids, w.weights, w.sorted_pairs, w.pair_pos, w.expert_offsets, w.chunk_hist,
                             logits, tokens, n_experts, top_k, 0, stream);
-    moe_quant_bf16_launcher(w.x_q, w.x_s, x, tokens, hidden, 0, stream);
+    moe_quant_bf16_launcher(w.x_q, w.x_s, x, tokens, hidden, config & CONFIG_UE8M0, stream);
     run_expert_gemms(w, w13_q, w13_s, w2_q, w2_s, tokens, hidden, inter, n_experts, top_k, config, stream);
     moe_combine_launcher(out, w.y, w.weights, w.pair_pos, tokens, hidden, top_k, out_dtype, 0, stream);
 }
@@ -264,7 +270,7 @@ extern "C" void moe_fp8_shared_launcher(void* out, const void* x, const float* l
     }
     moe_route_sort_launcher(w.ids, w.weights, w.sorted_pairs, w.pair_pos, w.expert_offsets, w.chunk_hist,
                             logits, tokens, n_experts, top_k, 0, stream);
-    moe_quant_bf16_launcher(w.x_q, w.x_s, x, tokens, hidden, 0, stream);
+    moe_quant_bf16_launcher(w.x_q, w.x_s, x, tokens, hidden, config & CONFIG_UE8M0, stream);
     run_expert_gemms(w, w13_q, w13_s, w2_q, w2_s, tokens, hidden, inter, n_experts, top_k, config, stream);
     sh.x_q = w.x_q;
     sh.x_s = w.x_s;

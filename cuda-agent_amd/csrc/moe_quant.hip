@@ -1,5 +1,6 @@
 // Activation quantisation: bf16 rows -> e4m3 codes with one fp32 scale per 128-wide group.
 //   scale = max(amax, 1e-12) * fp32(1/448);  code = e4m3_rne(clamp(v / scale, -448, 448))
+//   (or, on request, scale = the smallest power of two >= max(amax, 1e-12) / 448)
 // One wavefront per (row, group), two elements per lane. The division is IEEE fp32 so that the
 // codes are bit-identical to a CPU evaluation of the same formula; v_cvt_pk_fp8_f32 rounds to
 // nearest even but does not saturate (465 -> NaN), hence the clamp.
@@ -15,7 +16,7 @@ using namespace moe;
 __global__ __launch_bounds__(256) void moe_quant_bf16_kernel(const __hip_bfloat16* __restrict__ x,
                                                              uint8_t* __restrict__ q,
                                                              float* __restrict__ scales,
-                                                             long n_groups) {
+                                                             long n_groups, bool pow2) {
     const int lane = threadIdx.x & 63;
     const long g = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (g >= n_groups) return;
@@ -25,7 +26,7 @@ __global__ __launch_bounds__(256) void moe_quant_bf16_kernel(const __hip_bfloat1
     float amax = fmaxf(fabsf(v0), fabsf(v1));
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
-    const float scale = fmaxf(amax, AMAX_FLOOR) * INV_E4M3_MAX;
+    const float scale = group_scale(amax, pow2);
     const float a = fminf(fmaxf(v0 / scale, -E4M3_MAX), E4M3_MAX);
     const float b = fminf(fmaxf(v1 / scale, -E4M3_MAX), E4M3_MAX);
     const int packed = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
@@ -37,7 +38,7 @@ __global__ __launch_bounds__(256) void moe_quant_bf16_kernel(const __hip_bfloat1
 __global__ __launch_bounds__(256) void moe_quant_bf16_vec_kernel(const __hip_bfloat16* __restrict__ x,
                                                                  uint8_t* __restrict__ q,
                                                                  float* __restrict__ scales,
-                                                                 long n_groups) {
+                                                                 long n_groups, bool pow2) {
     typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
     typedef unsigned uintx2 __attribute__((ext_vector_type(2)));
     const int sub = threadIdx.x & 15;
@@ -55,7 +56,7 @@ __global__ __launch_bounds__(256) void moe_quant_bf16_vec_kernel(const __hip_bfl
     for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
 #pragma unroll
     for (int off = 8; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
-    const float scale = fmaxf(amax, AMAX_FLOOR) * INV_E4M3_MAX;
+    const float scale = group_scale(amax, pow2);
 #pragma unroll
     for (int j = 0; j < 8; ++j) v[j] = fminf(fmaxf(v[j] / scale, -E4M3_MAX), E4M3_MAX);
     uintx2 packed;
@@ -72,9 +73,10 @@ __global__ __launch_bounds__(256) void moe_quant_bf16_vec_kernel(const __hip_bfl
 }  // namespace
 
 // q [rows, cols] e4m3 codes and scales [rows, cols/128] fp32 from x [rows, cols] bf16.
+// config bit 32: power-of-two scales (the smallest power of two >= amax / 448).
 extern "C" void moe_quant_bf16_launcher(void* q, float* scales, const void* x, int rows, int cols,
                                         int config, hipStream_t stream) {
-    (void)config;
+    const bool pow2 = (config & CONFIG_UE8M0) != 0;
     if (rows <= 0 || cols <= 0) return;
     if (cols % GROUP != 0) {
         caa::set_status(CAA_UNSUPPORTED_SHAPE);
@@ -88,10 +90,10 @@ extern "C" void moe_quant_bf16_launcher(void* q, float* scales, const void* x, i
     const long n_groups = (long)rows * (cols / GROUP);
     if (!(reinterpret_cast<uintptr_t>(x) & 15u) && !(reinterpret_cast<uintptr_t>(q) & 7u)) {
         moe_quant_bf16_vec_kernel<<<dim3((unsigned)((n_groups + 15) / 16)), 256, 0, stream>>>(
-            static_cast<const __hip_bfloat16*>(x), static_cast<uint8_t*>(q), scales, n_groups);
+            static_cast<const __hip_bfloat16*>(x), static_cast<uint8_t*>(q), scales, n_groups, pow2);
         return;
     }
     const long blocks = (n_groups + 3) / 4;
     moe_quant_bf16_kernel<<<dim3((unsigned)blocks), 256, 0, stream>>>(
-        static_cast<const __hip_bfloat16*>(x), static_cast<uint8_t*>(q), scales, n_groups);
+        static_cast<const __hip_bfloat16*>(x), static_cast<uint8_t*>(q), scales, n_groups, pow2);
 }

@@ -257,7 +257,10 @@ void moe_fp8_workspace_layout(size_t* offsets10, int tokens, int hidden, int int
  * aligned. hidden and inter multiples of 128. config: 0 picks the GEMM form from the average number
  * of pairs per expert (above 32 and hidden % 256 == 0: LDS-tiled 256x256 GEMMs; otherwise the
  * weight-streaming form); 16 forces the tiled form; 1, 2, 4 (+8) force streaming as for
- * moe_gate_up_launcher. */
+ * moe_gate_up_launcher. +32 (also understood by moe_quant_bf16_launcher and moe_gate_up_launcher):
+ * every block scale is a power of two (UE8M0). w13_s and w2_s must then hold powers of two; x and
+ * the intermediate are quantised with scale = the smallest power of two >= max(amax, 1e-12)/448,
+ * and the tiled GEMMs apply the scales inside the MFMA. */
 void moe_fp8_launcher(void* out, const void* x, const float* logits, const void* w13_q,
                       const float* w13_s, const void* w2_q, const float* w2_s, void* workspace,
                       size_t workspace_bytes, int tokens, int hidden, int inter, int n_experts,

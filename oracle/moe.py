@@ -32,6 +32,13 @@ product and by the same fixture's logits.
 ``moe_forward_shared`` adds the shared expert of such a layer; it is built from ``moe_forward`` itself
 and pinned by a float64 dense evaluation of the same sum on a tiny shape.
 
+The UE8M0 form of the layer (``pow2_scales``; no counterpart in the reference repository) changes one
+line of the specification: an activation scale is the smallest power of two >= amax/448 instead of
+amax * fp32(1/448); weight scales are given as powers of two. Pinned by: ``pow2_ceil`` against float64
+``2**ceil(log2 v)`` and on exact powers of two and their neighbours; scale in [amax/448, 2*amax/448);
+the group maximum maps to a code in [224, 448]; division by the scale exact (codes equal the e4m3
+rounding of an exactly scaled value); the dense float64 layer evaluation with those scales.
+
 Pinned by (tests/test_oracle_moe.py):
   * e4m3: the 256-entry decode table against torch's float8_e4m3fn and the closed form; the
     encoder against torch's cast on every representable value, every midpoint and random
@@ -91,13 +98,28 @@ def e4m3_encode(x):
     return code.astype(np.uint8)
 
 
-def quantize_groups(v):
+def pow2_ceil(v):
+    """The smallest power of two >= v, for positive fp32 v, exactly (frexp: v = m * 2^e, 0.5 <= m < 1)."""
+    m, e = torch.frexp(v.float())
+    return torch.ldexp(torch.ones_like(m), torch.where(m == 0.5, e - 1, e))
+
+
+def quantize_groups(v, pow2=False):
     """Per-row, per-128-group e4m3 quantisation of a 2-D fp32 tensor.
-    Returns (codes float8_e4m3fn [R,C], scales fp32 [R,C/128])."""
+    Returns (codes float8_e4m3fn [R,C], scales fp32 [R,C/128]). ``pow2``: the UE8M0 convention, scale =
+    the smallest power of two >= amax/448."""
     R, C = v.shape
     g = v.float().reshape(R, C // GROUP, GROUP)
     amax = g.abs().amax(dim=-1).clamp_min(AMAX_FLOOR)
-    scale = amax * (1.0 / E4M3_MAX)
+    if pow2:
+        # amax/448 in float64 is not exact, but a power of two p satisfies p >= amax/448 iff 448*p >= amax,
+        # and 448*p is exact: take the candidate from the rounded quotient and correct it by one step
+        p = pow2_ceil((amax.double() / E4M3_MAX).float())
+        p = torch.where(p.double() * E4M3_MAX < amax.double(), p * 2, p)
+        p = torch.where((p.double() / 2) * E4M3_MAX >= amax.double(), p / 2, p)
+        scale = p
+    else:
+        scale = amax * (1.0 / E4M3_MAX)
     q = (g / scale[:, :, None]).clamp(-E4M3_MAX, E4M3_MAX).to(torch.float8_e4m3fn)
     return q.reshape(R, C), scale
 
@@ -173,12 +195,17 @@ def silu(x):
 
 
 def moe_forward(x, logits, w13_q, w13_s, w2_q, w2_s, top_k=8, out_dtype=torch.bfloat16,
-                return_intermediates=False):
+                return_intermediates=False, pow2_scales=False):
+    """``pow2_scales``: the UE8M0 form of the layer, activations quantised with power-of-two scales (the
+    weight scales handed in must be powers of two as well; checked)."""
+    if pow2_scales:
+        for ws in (w13_s, w2_s):
+            assert torch.equal(ws, pow2_ceil(ws)), 'UE8M0 form: weight scales must be powers of two'
     T, H = x.shape
     E, I2, _ = w13_q.shape
     I = I2 // 2
     ids, weights = route(logits, top_k)
-    x_q, x_s = quantize_groups(x.float())
+    x_q, x_s = quantize_groups(x.float(), pow2_scales)
     x_dq = dequantize_groups(x_q, x_s)
     y = torch.zeros(T, top_k, H)
     h_q_all = torch.zeros(T, top_k, I, dtype=torch.float8_e4m3fn)
@@ -188,7 +215,7 @@ def moe_forward(x, logits, w13_q, w13_s, w2_q, w2_s, top_k=8, out_dtype=torch.bf
         w13 = dequantize_blocks(w13_q[e], w13_s[e])
         gu = x_dq[tok] @ w13.T
         h = silu(gu[:, :I]) * gu[:, I:]
-        h_q, h_s = quantize_groups(h)
+        h_q, h_s = quantize_groups(h, pow2_scales)
         h_q_all[tok, slot] = h_q
         h_s_all[tok, slot] = h_s
         y[tok, slot] = dequantize_groups(h_q, h_s) @ dequantize_blocks(w2_q[e], w2_s[e]).T
@@ -202,14 +229,14 @@ def moe_forward(x, logits, w13_q, w13_s, w2_q, w2_s, top_k=8, out_dtype=torch.bf
 
 
 def moe_forward_shared(x, logits, w13_q, w13_s, w2_q, w2_s, sw13_q, sw13_s, sw2_q, sw2_s, top_k=8,
-                       out_dtype=torch.bfloat16):
+                       out_dtype=torch.bfloat16, pow2_scales=False):
     """The layer plus a shared expert: one more block-scaled MLP (sw13_q [2*Is,H], sw13_s, sw2_q [H,Is],
     sw2_s) applied to every token with weight 1, added in fp32 after the routed experts' weighted sum.
     The shared expert is evaluated by the same stage functions: a layer of one expert chosen by every
     token with routing weight s/s = 1."""
-    routed = moe_forward(x, logits, w13_q, w13_s, w2_q, w2_s, top_k, torch.float32)
+    routed = moe_forward(x, logits, w13_q, w13_s, w2_q, w2_s, top_k, torch.float32, pow2_scales=pow2_scales)
     shared = moe_forward(x, torch.zeros(x.shape[0], 1), sw13_q[None], sw13_s[None], sw2_q[None], sw2_s[None],
-                         1, torch.float32)
+                         1, torch.float32, pow2_scales=pow2_scales)
     return (routed + shared).to(out_dtype)
 
 
@@ -229,10 +256,11 @@ def normal_e4m3(shape, std, generator=None, device='cpu'):
     return v.clamp(-E4M3_MAX, E4M3_MAX).to(torch.float8_e4m3fn)
 
 
-def moe_make_weights(n_experts, hidden, inter, generator=None, device='cpu'):
+def moe_make_weights(n_experts, hidden, inter, generator=None, device='cpu', pow2_scales=False):
     """Expert weights: e4m3 codes of N(0, 448/sqrt(fan_in)) and 128x128 block scales
     ~ U(0.5, 1.5)/448, so that a dequantised weight is about N(0, 1/fan_in) and the
-    pre-activations of N(0,1) inputs are O(1). (The workload leaves the code distribution open.)"""
+    pre-activations of N(0,1) inputs are O(1). (The workload leaves the code distribution open.)
+    ``pow2_scales``: every scale rounded up to a power of two (2^-9 or 2^-8)."""
     gen = generator
     w13_q = normal_e4m3((n_experts, 2 * inter, hidden), E4M3_MAX / hidden ** 0.5, gen, device)
     w2_q = normal_e4m3((n_experts, hidden, inter), E4M3_MAX / inter ** 0.5, gen, device)
@@ -240,6 +268,8 @@ def moe_make_weights(n_experts, hidden, inter, generator=None, device='cpu'):
                               device=device)) / 448.0
     w2_s = (0.5 + torch.rand(n_experts, hidden // GROUP, inter // GROUP, generator=gen,
                              device=device)) / 448.0
+    if pow2_scales:
+        w13_s, w2_s = pow2_ceil(w13_s), pow2_ceil(w2_s)
     return w13_q, w13_s, w2_q, w2_s
 
 

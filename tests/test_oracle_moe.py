@@ -288,3 +288,64 @@ def test_router_logits_against_float64_and_golden():
     for tag in 'abc':
         got = moe.router_logits(torch.from_numpy(z[f'{tag}_hidden']).bfloat16(), torch.from_numpy(z[f'{tag}_weight']))
         torch.testing.assert_close(got, torch.from_numpy(z[f'{tag}_logits']), rtol=1e-5, atol=1e-6)
+
+
+# ---- power-of-two (UE8M0) scales -----------------------------------------------------------------
+
+def test_pow2_ceil_is_exact():
+    gen = torch.Generator().manual_seed(61)
+    v = torch.exp(torch.randn(4000, generator=gen) * 8).float()
+    want = torch.pow(2.0, torch.ceil(torch.log2(v.double())))
+    assert torch.equal(moe.pow2_ceil(v).double(), want)
+    p = torch.ldexp(torch.ones(60), torch.arange(-30, 30))
+    assert torch.equal(moe.pow2_ceil(p), p)
+    assert torch.equal(moe.pow2_ceil(torch.nextafter(p, torch.full_like(p, float('inf')))), 2 * p)
+    assert torch.equal(moe.pow2_ceil(torch.nextafter(p, torch.zeros_like(p))), p)
+
+
+def test_pow2_group_quantisation_properties():
+    gen = torch.Generator().manual_seed(62)
+    v = torch.randn(64, 512, generator=gen) * torch.exp(torch.randn(64, 1, generator=gen) * 3)
+    v[3, :128] = 0.0                                   # an all-zero group takes the floor
+    v[4, 5] = 448.0 * 2 ** -3                          # amax/448 exactly a power of two
+    v[4, :128] = v[4, :128].clamp(-56.0, 56.0)
+    v[5, 130] = float(torch.nextafter(torch.tensor(448.0 * 4), torch.tensor(1e9)))   # just above
+    v[5, 128:256] = v[5, 128:256].clamp(-1793.0, 1793.0)
+    q, s = moe.quantize_groups(v, pow2=True)
+    assert torch.equal(s, moe.pow2_ceil(s))                                  # powers of two
+    amax = v.reshape(64, 4, 128).abs().amax(dim=-1).clamp_min(moe.AMAX_FLOOR).double()
+    assert (s.double() * 448 >= amax).all() and (s.double() * 224 < amax).all()
+    assert s[4, 0] == 2 ** -3 and s[5, 1] == 8.0
+    # the division is exact, so the codes are the e4m3 rounding of v / s computed in float64
+    want = (v.double().reshape(64, 4, 128) / s.double()[:, :, None]).float().to(torch.float8_e4m3fn)
+    assert torch.equal(q.view(torch.uint8), want.reshape(64, 512).view(torch.uint8))
+    top = q.float().reshape(64, 4, 128).abs().amax(dim=-1)
+    live = amax > moe.AMAX_FLOOR
+    assert (top[live] >= 224).all() and (top <= 448).all()      # amax/s in (224, 448] rounds to a code >= 224
+    # idempotent on its own output
+    dq = moe.dequantize_groups(q, s)
+    q2, _ = moe.quantize_groups(dq, pow2=True)
+    assert torch.equal(moe.dequantize_groups(q2, moe.quantize_groups(dq, pow2=True)[1]), dq)
+
+
+def test_pow2_layer_against_float64_dense():
+    gen = torch.Generator().manual_seed(63)
+    w13_q, w13_s, w2_q, w2_s = moe.moe_make_weights(4, 256, 128, gen, pow2_scales=True)
+    x, logits = moe.moe_make_inputs(8, 256, 4, gen)
+    out, mid = moe.moe_forward(x, logits, w13_q, w13_s, w2_q, w2_s, top_k=2, out_dtype=torch.float32,
+                               return_intermediates=True, pow2_scales=True)
+    assert torch.equal(mid['x_s'], moe.pow2_ceil(mid['x_s'])) and torch.equal(mid['h_s'], moe.pow2_ceil(mid['h_s']))
+    ids, wts = mid['ids'], mid['weights'].double()
+    xd = moe.dequantize_groups(mid['x_q'], mid['x_s']).double()
+    want = torch.zeros(8, 256, dtype=torch.float64)
+    for t in range(8):
+        for k in range(2):
+            e = ids[t, k].item()
+            gu = moe.dequantize_blocks(w13_q[e], w13_s[e]).double() @ xd[t]
+            h = gu[:128] / (1 + torch.exp(-gu[:128])) * gu[128:]
+            hq, hs = moe.quantize_groups(h.float()[None], pow2=True)
+            want[t] += wts[t, k] * (moe.dequantize_blocks(w2_q[e], w2_s[e]).double()
+                                    @ moe.dequantize_groups(hq, hs)[0].double())
+    assert moe.rel_rms_error(out, want) < 1e-4
+    with pytest.raises(AssertionError):
+        moe.moe_forward(x, logits, w13_q, w13_s * 1.5, w2_q, w2_s, top_k=2, pow2_scales=True)
