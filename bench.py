@@ -305,20 +305,28 @@ def bench_mla(torch, capi, dev, steps, warmup, cpu_baseline, paged=False):
 
 
 def make_moe(torch, dev, tokens, biased):
+    """The workload's tensors. The weight buffers hold one more expert behind the 256 routed ones (the shared
+    expert of the `with_shared_expert` timings, seed 20258); the routed experts are views of the first 256."""
     H, I, E = 7168, 2048, 256
     gen = torch.Generator(device=dev).manual_seed(20252 if not biased else 20254)
-    w13_q = torch.empty(E, 2 * I, H, dtype=torch.float8_e4m3fn, device=dev)
-    w2_q = torch.empty(E, H, I, dtype=torch.float8_e4m3fn, device=dev)
+    w13_all = torch.empty(E + 1, 2 * I, H, dtype=torch.float8_e4m3fn, device=dev)
+    w2_all = torch.empty(E + 1, H, I, dtype=torch.float8_e4m3fn, device=dev)
     for e in range(E):
-        w13_q[e] = (torch.randn(2 * I, H, device=dev, generator=gen) * (448 / H ** 0.5)).to(torch.float8_e4m3fn)
-        w2_q[e] = (torch.randn(H, I, device=dev, generator=gen) * (448 / I ** 0.5)).to(torch.float8_e4m3fn)
+        w13_all[e] = (torch.randn(2 * I, H, device=dev, generator=gen) * (448 / H ** 0.5)).to(torch.float8_e4m3fn)
+        w2_all[e] = (torch.randn(H, I, device=dev, generator=gen) * (448 / I ** 0.5)).to(torch.float8_e4m3fn)
     w13_s = (0.5 + torch.rand(E, 2 * I // 128, H // 128, device=dev, generator=gen)) / 448
     w2_s = (0.5 + torch.rand(E, H // 128, I // 128, device=dev, generator=gen)) / 448
     x = torch.randn(tokens, H, device=dev, generator=gen).bfloat16()
     logits = torch.randn(tokens, E, device=dev, generator=gen)
     if biased:
         logits[:, torch.randperm(E, device=dev, generator=gen)[:16]] += 2.0
-    return x, logits, w13_q, w13_s, w2_q, w2_s
+    gen = torch.Generator(device=dev).manual_seed(20258)
+    w13_all[E] = (torch.randn(2 * I, H, device=dev, generator=gen) * (448 / H ** 0.5)).to(torch.float8_e4m3fn)
+    w2_all[E] = (torch.randn(H, I, device=dev, generator=gen) * (448 / I ** 0.5)).to(torch.float8_e4m3fn)
+    w13_s_all = torch.cat([w13_s, ((0.5 + torch.rand(1, 2 * I // 128, H // 128, device=dev, generator=gen)) / 448)])
+    w2_s_all = torch.cat([w2_s, ((0.5 + torch.rand(1, H // 128, I // 128, device=dev, generator=gen)) / 448)])
+    stacked = (w13_all, w13_s_all, w2_all, w2_s_all)
+    return (x, logits, w13_all[:E], w13_s, w2_all[:E], w2_s), stacked
 
 
 def moe_cpu_baseline(torch, tensors, n_tokens):
@@ -342,7 +350,7 @@ def moe_cpu_baseline(torch, tensors, n_tokens):
 def bench_moe(torch, capi, dev, steps, warmup, cpu_baseline, prefill):
     T = 8192 if prefill else 64
     H, I, E, k = 7168, 2048, 256, 8
-    tensors = make_moe(torch, dev, T, prefill)
+    tensors, stacked = make_moe(torch, dev, T, prefill)
     x, logits, w13_q, w13_s, w2_q, w2_s = tensors
     ws = torch.empty(capi.moe_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device=dev)
     out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
@@ -370,23 +378,27 @@ def bench_moe(torch, capi, dev, steps, warmup, cpu_baseline, prefill):
             roofline=dict(bound="hbm", achieved=wbytes / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
                           frac=wbytes / sec / 1e9 / HBM_PEAK_GBS, traffic=MEASURED_TRAFFIC['moe_decode']),
             algorithmic_bytes=wbytes, active_experts=n_active, tflops=flops / sec / 1e12)
-    # the same layer with a shared expert (one more block-scaled MLP of inter 2048 on every token)
-    gen = torch.Generator(device=dev).manual_seed(20258)
-    sw13_q = (torch.randn(2 * I, H, device=dev, generator=gen) * (448 / H ** 0.5)).to(torch.float8_e4m3fn)
-    sw2_q = (torch.randn(H, I, device=dev, generator=gen) * (448 / I ** 0.5)).to(torch.float8_e4m3fn)
-    sw13_s = (0.5 + torch.rand(2 * I // 128, H // 128, device=dev, generator=gen)) / 448
-    sw2_s = (0.5 + torch.rand(H // 128, I // 128, device=dev, generator=gen)) / 448
+    # the same layer with a shared expert (one more block-scaled MLP of inter 2048 on every token): as launches
+    # of its own, and stored behind the routed experts so that it runs inside their launches
+    sw13_q, sw13_s, sw2_q, sw2_s = (t[E] for t in stacked)
     del ws
     ws2 = torch.empty(capi.moe_shared_workspace_bytes(T, H, I, I, E, k), dtype=torch.uint8, device=dev)
     sec2 = timed_launches(
         torch, lambda i: capi.moe_fp8_shared_launch(out, x, logits, w13_q, w13_s, w2_q, w2_s, sw13_q, sw13_s,
                                                     sw2_q, sw2_s, ws2), steps, warmup)
+    del ws2
+    ws2 = torch.empty(capi.moe_workspace_bytes(T, H, I, E + 1, k + 1), dtype=torch.uint8, device=dev)
+    sec2f = timed_launches(torch, lambda i: capi.moe_fp8_fused_shared_launch(out, x, logits, *stacked, ws2),
+                           steps, warmup)
     flops2 = flops + T * (2 * H * 2 * I + 2 * I * H)
     wbytes2 = wbytes + 3 * I * H + (3 * I * H // (128 * 128)) * 4
     res['with_shared_expert'] = dict(
-        ms_per_step=sec2 * 1e3, unit=res['unit'],
-        value=flops2 / sec2 / 1e12 if prefill else wbytes2 / sec2 / 1e9,
-        note="moe_fp8_shared_launcher: the layer above plus one shared expert of inter 2048, seed 20258")
+        ms_per_step=sec2f * 1e3, unit=res['unit'],
+        value=flops2 / sec2f / 1e12 if prefill else wbytes2 / sec2f / 1e9,
+        ms_per_step_separate_launches=sec2 * 1e3,
+        note="the layer above plus one shared expert of inter 2048, seed 20258: moe_fp8_fused_shared_launcher "
+             "(stored as expert 256, inside the routed experts' launches); ms_per_step_separate_launches is "
+             "moe_fp8_shared_launcher (its own launches)")
     del ws2
     # the same layer with power-of-two (UE8M0) block scales: the weight scales rounded up to powers of two,
     # activations quantised with power-of-two scales, the tiled GEMMs scaled by the MFMA itself

@@ -49,6 +49,8 @@ SIGNATURES = {
     'moe_fp8_shared_workspace_bytes': (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
     'moe_fp8_shared_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int,
                                        c_int, c_int, c_int, c_int, c_int, c_int, _P]),
+    'moe_fp8_fused_shared_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int,
+                                             c_int, c_int, c_int, c_int, _P]),
     'moe_fp8_workspace_bytes': (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
     'moe_fp8_workspace_layout': (None, [_P, c_int, c_int, c_int, c_int, c_int]),
     'moe_fp8_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int,
@@ -451,3 +453,30 @@ def moe_fp8_shared_launch(out, x, logits, w13_q, w13_s, w2_q, w2_s, sw13_q, sw13
         T, H, I, Is, E, top_k, 0 if out.dtype == torch.bfloat16 else 1, config, _stream(stream))
     check_status('moe_fp8_shared_launcher')
     return out
+
+
+def moe_fp8_fused_shared_launch(out, x, logits, w13_q, w13_s, w2_q, w2_s, workspace, top_k=8, config=0,
+                                stream=None):
+    """The layer with the shared expert stored as the last of E+1 experts in the weight tensors; logits [T, E].
+    ``workspace``: ``moe_workspace_bytes(T, H, I, E + 1, top_k + 1)`` bytes."""
+    import torch
+    _device_contiguous(out=out, x=x, logits=logits, w13_q=w13_q, w13_s=w13_s, w2_q=w2_q, w2_s=w2_s,
+                       workspace=workspace)
+    T, H = x.shape
+    E1, I2, _ = w13_q.shape
+    I, E = I2 // 2, E1 - 1
+    _require(x.dtype == torch.bfloat16 and logits.dtype == torch.float32, 'moe_fp8: x bf16, logits fp32')
+    _require(out.dtype in (torch.bfloat16, torch.float32) and tuple(out.shape) == (T, H), 'moe_fp8: out')
+    _require(w13_q.element_size() == 1 and w2_q.element_size() == 1, 'moe_fp8: weights must be e4m3')
+    _require(tuple(w13_q.shape) == (E1, 2 * I, H) and tuple(w2_q.shape) == (E1, H, I), 'moe_fp8: weight shapes')
+    _require(tuple(w13_s.shape) == (E1, 2 * I // 128, H // 128) and tuple(w2_s.shape) == (E1, H // 128, I // 128),
+             'moe_fp8: scale shapes')
+    _require(w13_s.dtype == torch.float32 and w2_s.dtype == torch.float32, 'moe_fp8: scales fp32')
+    _require(tuple(logits.shape) == (T, E), 'moe_fp8: logits [T, E] for E + 1 stored experts')
+    library().moe_fp8_fused_shared_launcher(
+        _ptr(out), _ptr(x), _ptr(logits), _ptr(w13_q), _ptr(w13_s), _ptr(w2_q), _ptr(w2_s), _ptr(workspace),
+        workspace.numel() * workspace.element_size(), T, H, I, E, top_k,
+        0 if out.dtype == torch.bfloat16 else 1, config, _stream(stream))
+    check_status('moe_fp8_fused_shared_launcher')
+    return out
+

@@ -18,6 +18,15 @@ constexpr int SORT_CHUNK_TOKENS = 256;
 // activation scales become the smallest power of two >= amax / 448.
 constexpr int CONFIG_UE8M0 = 32;
 
+// config bit of the routing launchers: every token gets one more slot after its top_k, expert number
+// n_experts with weight 1 (a shared expert stored as one more expert behind the routed ones); ids and
+// weights then have top_k + 1 entries per token and the sort covers n_experts + 1 experts.
+constexpr int CONFIG_SHARED_SLOT = 64;
+
+// config bit of the streaming GEMM launchers (and of the layer's internal calls): the last expert holds far
+// more pairs than the others (the shared expert above): dispatch its workgroups first.
+constexpr int CONFIG_LAST_EXPERT_FIRST = 128;
+
 #ifdef __HIPCC__
 // scale of a 128-wide activation group with maximum magnitude amax
 __device__ __forceinline__ float group_scale(float amax, bool pow2) {

@@ -45,11 +45,14 @@ __global__ __launch_bounds__(256) void moe_stream_gemm_kernel(
     const uint8_t* __restrict__ w_q, const float* __restrict__ w_s, const uint8_t* __restrict__ a_q,
     const float* __restrict__ a_s, const int* __restrict__ sorted_pairs,
     const int* __restrict__ expert_offsets, uint8_t* __restrict__ h_q, float* __restrict__ h_s,
-    float* __restrict__ y, int K, int n_rows, int inter, int top_k, bool pow2) {
+    float* __restrict__ y, int K, int n_rows, int inter, int top_k, bool pow2,
+    bool last_first) {
     constexpr int TILES = GATE_UP ? 4 : 2;
     __shared__ float s_amax[4][NT * 16];
 
-    const int e = blockIdx.y;
+    // last_first: the last expert is the heaviest (a shared expert that every token uses): its
+    // workgroups are dispatched first, so that its several passes do not become the launch's tail
+    const int e = last_first ? (blockIdx.y == 0 ? (int)gridDim.y - 1 : (int)blockIdx.y - 1) : (int)blockIdx.y;
     const int rb = blockIdx.x;  // 128-row block of the output dimension
     const int begin = expert_offsets[e];
     const int end = expert_offsets[e + 1];
@@ -243,7 +246,8 @@ __global__ __launch_bounds__(256) void moe_stream_gemm_lds_kernel(
     const uint8_t* __restrict__ w_q, const float* __restrict__ w_s, const uint8_t* __restrict__ a_q,
     const float* __restrict__ a_s, const int* __restrict__ sorted_pairs,
     const int* __restrict__ expert_offsets, uint8_t* __restrict__ h_q, float* __restrict__ h_s,
-    float* __restrict__ y, int K, int n_rows, int inter, int top_k, bool pow2) {
+    float* __restrict__ y, int K, int n_rows, int inter, int top_k, bool pow2,
+    bool last_first) {
     constexpr int TILES = 4;
     constexpr int DEPTH = 3;
     constexpr int TILE_BYTES = 16 * GROUP;                       // 2 KB
@@ -254,7 +258,9 @@ __global__ __launch_bounds__(256) void moe_stream_gemm_lds_kernel(
     __shared__ float s_bscale[MAX_KB][NT * 16];
     __shared__ float s_amax[4][NT * 16];
 
-    const int e = blockIdx.y;
+    // last_first: the last expert is the heaviest (a shared expert that every token uses): its
+    // workgroups are dispatched first, so that its several passes do not become the launch's tail
+    const int e = last_first ? (blockIdx.y == 0 ? (int)gridDim.y - 1 : (int)blockIdx.y - 1) : (int)blockIdx.y;
     const int rb = blockIdx.x;  // block of 256 output rows (GATE_UP: 128 gate + 128 up)
     const int begin = expert_offsets[e];
     const int end = expert_offsets[e + 1];
@@ -477,7 +483,8 @@ extern "C" void moe_gate_up_launcher(void* h_q, float* h_s, const void* x_q, con
     const auto* xq = static_cast<const uint8_t*>(x_q);
     const auto* wq = static_cast<const uint8_t*>(w13_q);
     const bool pow2 = (config & CONFIG_UE8M0) != 0;
-    config &= ~CONFIG_UE8M0;
+    const bool last_first = (config & CONFIG_LAST_EXPERT_FIRST) != 0;
+    config &= ~(CONFIG_UE8M0 | CONFIG_LAST_EXPERT_FIRST);
     int nt = config & 7;
     if (nt != 1 && nt != 2 && nt != 4) {
         const long avg = (long)tokens * top_k / n_experts;  // pairs per expert if spread evenly
@@ -489,28 +496,28 @@ extern "C" void moe_gate_up_launcher(void* h_q, float* h_s, const void* x_q, con
             if (lds_path) {
                 moe_stream_gemm_lds_kernel<true, 1><<<grid, 256, 0, stream>>>(
                     wq, w13_s, xq, x_s, sorted_pairs, expert_offsets, hq, h_s, nullptr, hidden,
-                    2 * inter, inter, top_k, pow2);
+                    2 * inter, inter, top_k, pow2, last_first);
             } else {
                 moe_stream_gemm_kernel<true, 1><<<grid, 256, 0, stream>>>(
                     wq, w13_s, xq, x_s, sorted_pairs, expert_offsets, hq, h_s, nullptr, hidden,
-                    2 * inter, inter, top_k, pow2);
+                    2 * inter, inter, top_k, pow2, last_first);
             }
             break;
         case 2:
             if (lds_path) {
                 moe_stream_gemm_lds_kernel<true, 2><<<grid, 256, 0, stream>>>(
                     wq, w13_s, xq, x_s, sorted_pairs, expert_offsets, hq, h_s, nullptr, hidden,
-                    2 * inter, inter, top_k, pow2);
+                    2 * inter, inter, top_k, pow2, last_first);
             } else {
                 moe_stream_gemm_kernel<true, 2><<<grid, 256, 0, stream>>>(
                     wq, w13_s, xq, x_s, sorted_pairs, expert_offsets, hq, h_s, nullptr, hidden,
-                    2 * inter, inter, top_k, pow2);
+                    2 * inter, inter, top_k, pow2, last_first);
             }
             break;
         default:
             moe_stream_gemm_kernel<true, 4><<<grid, 256, 0, stream>>>(
                 wq, w13_s, xq, x_s, sorted_pairs, expert_offsets, hq, h_s, nullptr, hidden, 2 * inter,
-                inter, top_k, pow2);
+                inter, top_k, pow2, last_first);
             break;
     }
 }
@@ -535,7 +542,9 @@ extern "C" void moe_down_launcher(float* y, const void* h_q, const float* h_s, c
     const dim3 grid(hidden / GROUP, n_experts);
     const auto* hq = static_cast<const uint8_t*>(h_q);
     const auto* wq = static_cast<const uint8_t*>(w2_q);
-    config &= ~CONFIG_UE8M0;  // (the down GEMM has no requantisation: nothing depends on the scale convention)
+    const bool last_first = (config & CONFIG_LAST_EXPERT_FIRST) != 0;
+    // (the down GEMM has no requantisation: nothing depends on the scale convention)
+    config &= ~(CONFIG_UE8M0 | CONFIG_LAST_EXPERT_FIRST);
     int nt = config & 7;
     if (nt != 1 && nt != 2 && nt != 4) {
         const long avg = (long)tokens * top_k / n_experts;
@@ -548,28 +557,28 @@ extern "C" void moe_down_launcher(float* y, const void* h_q, const float* h_s, c
             if (lds_path) {
                 moe_stream_gemm_lds_kernel<false, 1><<<grid256, 256, 0, stream>>>(
                     wq, w2_s, hq, h_s, nullptr, expert_offsets, nullptr, nullptr, y, inter, hidden,
-                    inter, top_k, false);
+                    inter, top_k, false, last_first);
             } else {
                 moe_stream_gemm_kernel<false, 1><<<grid, 256, 0, stream>>>(
                     wq, w2_s, hq, h_s, nullptr, expert_offsets, nullptr, nullptr, y, inter, hidden,
-                    inter, top_k, false);
+                    inter, top_k, false, last_first);
             }
             break;
         case 2:
             if (lds_path) {
                 moe_stream_gemm_lds_kernel<false, 2><<<grid256, 256, 0, stream>>>(
                     wq, w2_s, hq, h_s, nullptr, expert_offsets, nullptr, nullptr, y, inter, hidden,
-                    inter, top_k, false);
+                    inter, top_k, false, last_first);
             } else {
                 moe_stream_gemm_kernel<false, 2><<<grid, 256, 0, stream>>>(
                     wq, w2_s, hq, h_s, nullptr, expert_offsets, nullptr, nullptr, y, inter, hidden,
-                    inter, top_k, false);
+                    inter, top_k, false, last_first);
             }
             break;
         default:
             moe_stream_gemm_kernel<false, 4><<<grid, 256, 0, stream>>>(
                 wq, w2_s, hq, h_s, nullptr, expert_offsets, nullptr, nullptr, y, inter, hidden, inter,
-                top_k, false);
+                top_k, false, last_first);
             break;
     }
 }

@@ -164,7 +164,8 @@ void run_expert_gemms(const moe::Workspace& w, const void* w13_q, const float* w
                       const void* w2_q, const float* w2_s, int tokens, int hidden, int inter,
                       int n_experts, int top_k, int config, hipStream_t stream) {
     const int ue8m0 = config & CONFIG_UE8M0;  // power-of-two block scales, see moe_fp8_launcher
-    config &= ~CONFIG_UE8M0;
+    const int order = config & CONFIG_LAST_EXPERT_FIRST;
+    config &= ~(CONFIG_UE8M0 | CONFIG_LAST_EXPERT_FIRST);
     // (the tiled kernels address activations with 32-bit byte offsets)
     const bool fits32 = (unsigned long long)tokens * hidden < (1ull << 32) &&
                         (unsigned long long)tokens * top_k * inter < (1ull << 32);
@@ -180,9 +181,9 @@ void run_expert_gemms(const moe::Workspace& w, const void* w13_q, const float* w
                                 hidden, inter, n_experts, top_k, w.scale_stride, ue8m0, stream);
     } else {
         moe_gate_up_launcher(w.h_q, w.h_s, w.x_q, w.x_s, w13_q, w13_s, w.sorted_pairs, w.expert_offsets,
-                             tokens, hidden, inter, n_experts, top_k, config | ue8m0, stream);
+                             tokens, hidden, inter, n_experts, top_k, config | ue8m0 | order, stream);
         moe_down_launcher(w.y, w.h_q, w.h_s, w2_q, w2_s, w.expert_offsets, tokens, hidden, inter,
-                          n_experts, top_k, config, stream);
+                          n_experts, top_k, config | order, stream);
     }
 }
 
@@ -280,3 +281,41 @@ extern "C" void moe_fp8_shared_launcher(void* out, const void* x, const float* l
     moe_combine_shared_launcher(out, w.y, w.weights, w.pair_pos, sh.y, tokens, hidden, top_k, out_dtype,
                                 0, stream);
 }
+
+// The layer with a shared expert stored as expert number n_experts behind the routed ones
+// (w13_q [n_experts + 1, 2*inter, hidden] and so on; same inter): every token takes it as one more
+// slot with weight 1 after its top_k, so it runs inside the routed experts' launches instead of as
+// under-filled launches of its own. out = sum_k w[t,k] * expert_k(x[t]) + expert_{n_experts}(x[t]),
+// the same sum as moe_fp8_shared_launcher. workspace: moe_fp8_workspace_bytes(tokens, hidden,
+// inter, n_experts + 1, top_k + 1) bytes with the layout of that shape. logits [tokens, n_experts].
+extern "C" void moe_fp8_fused_shared_launcher(void* out, const void* x, const float* logits,
+                                              const void* w13_q, const float* w13_s,
+                                              const void* w2_q, const float* w2_s, void* workspace,
+                                              size_t workspace_bytes, int tokens, int hidden,
+                                              int inter, int n_experts, int top_k, int out_dtype,
+                                              int config, hipStream_t stream) {
+    if (tokens <= 0) return;
+    if (!layer_shape_ok(hidden, inter, n_experts, top_k, tokens, out_dtype) || n_experts >= 512 ||
+        top_k >= 64 || (long)tokens * (top_k + 1) > 0x7fffffffL / 4) {
+        caa::set_status(CAA_UNSUPPORTED_SHAPE);
+        return;
+    }
+    if (!out || !x || !logits || !w13_q || !w13_s || !w2_q || !w2_s || !workspace ||
+        (reinterpret_cast<uintptr_t>(workspace) & 255u)) {
+        caa::set_status(CAA_BAD_ARGUMENT);
+        return;
+    }
+    const moe::Workspace w =
+        moe::carve_workspace(workspace, tokens, hidden, inter, n_experts + 1, top_k + 1);
+    if (workspace_bytes < w.bytes) {
+        caa::set_status(CAA_WORKSPACE_TOO_SMALL);
+        return;
+    }
+    moe_route_sort_launcher(w.ids, w.weights, w.sorted_pairs, w.pair_pos, w.expert_offsets, w.chunk_hist,
+                            logits, tokens, n_experts, top_k, CONFIG_SHARED_SLOT, stream);
+    moe_quant_bf16_launcher(w.x_q, w.x_s, x, tokens, hidden, config & CONFIG_UE8M0, stream);
+    run_expert_gemms(w, w13_q, w13_s, w2_q, w2_s, tokens, hidden, inter, n_experts + 1, top_k + 1,
+                     (config & ~CONFIG_LAST_EXPERT_FIRST) | CONFIG_LAST_EXPERT_FIRST, stream);
+    moe_combine_launcher(out, w.y, w.weights, w.pair_pos, tokens, hidden, top_k + 1, out_dtype, 0, stream);
+}
+

@@ -32,7 +32,10 @@ template <int PER_LANE>
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits,
                                                         int* __restrict__ ids,
                                                         float* __restrict__ weights, int tokens,
-                                                        int n_experts, int top_k) {
+                                                        int n_experts, int top_k, int shared) {
+    // shared == 1: every token gets one more slot, expert number n_experts with weight 1 (a shared
+    // expert stored behind the routed ones); rows of ids/weights then have top_k + 1 entries
+    const int slots = top_k + shared;
     const int lane = threadIdx.x & 63;
     const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (t >= tokens) return;
@@ -68,8 +71,11 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
         }
     }
     if (lane < top_k) {
-        ids[(size_t)t * top_k + lane] = my_id;
-        weights[(size_t)t * top_k + lane] = my_score / total;
+        ids[(size_t)t * slots + lane] = my_id;
+        weights[(size_t)t * slots + lane] = my_score / total;
+    } else if (lane == top_k && shared) {
+        ids[(size_t)t * slots + lane] = n_experts;
+        weights[(size_t)t * slots + lane] = 1.f;
     }
 }
 
@@ -351,13 +357,15 @@ template <int PER_LANE>
 __global__ __launch_bounds__(1024) void moe_route_sort_small_kernel(
     const float* __restrict__ logits, int* __restrict__ ids, float* __restrict__ weights,
     int* __restrict__ sorted_pairs, int* __restrict__ pair_pos, int* __restrict__ expert_offsets,
-    int tokens, int n_experts, int top_k) {
+    int tokens, int n_experts, int top_k, int shared) {
     __shared__ int s_ids[1024];
-    __shared__ int s_count[512 + 1];
+    __shared__ int s_count[512 + 2];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int pairs = tokens * top_k;
-    for (int e = threadIdx.x; e <= n_experts; e += 1024) s_count[e] = 0;
+    const int slots = top_k + shared;        // see moe_route_kernel
+    const int sorted_experts = n_experts + shared;
+    const int pairs = tokens * slots;
+    for (int e = threadIdx.x; e <= sorted_experts; e += 1024) s_count[e] = 0;
     for (int t = wave; t < tokens; t += 16) {
         unsigned long long key[PER_LANE];
 #pragma unroll
@@ -389,9 +397,13 @@ __global__ __launch_bounds__(1024) void moe_route_sort_small_kernel(
             }
         }
         if (lane < top_k) {
-            ids[(size_t)t * top_k + lane] = my_id;
-            weights[(size_t)t * top_k + lane] = my_score / total;
-            s_ids[t * top_k + lane] = my_id;
+            ids[(size_t)t * slots + lane] = my_id;
+            weights[(size_t)t * slots + lane] = my_score / total;
+            s_ids[t * slots + lane] = my_id;
+        } else if (lane == top_k && shared) {
+            ids[(size_t)t * slots + lane] = n_experts;
+            weights[(size_t)t * slots + lane] = 1.f;
+            s_ids[t * slots + lane] = n_experts;
         }
     }
     __syncthreads();
@@ -403,8 +415,8 @@ __global__ __launch_bounds__(1024) void moe_route_sort_small_kernel(
         for (int i = 0; i < p; ++i) rank += s_ids[i] == mine;
     }
     __syncthreads();
-    block_exclusive_scan(s_count, n_experts);  // in place; s_count[n_experts] = number of pairs
-    for (int e = threadIdx.x; e <= n_experts; e += 1024) expert_offsets[e] = s_count[e];
+    block_exclusive_scan(s_count, sorted_experts);  // in place; s_count[sorted_experts] = number of pairs
+    for (int e = threadIdx.x; e <= sorted_experts; e += 1024) expert_offsets[e] = s_count[e];
     if (p < pairs) {
         const int pos = s_count[mine] + rank;
         sorted_pairs[pos] = p;
@@ -424,9 +436,10 @@ extern "C" void moe_route_sort_launcher(int* ids, float* weights, int* sorted_pa
 // ids [tokens, top_k] int32 and weights [tokens, top_k] fp32 from logits [tokens, n_experts] fp32.
 extern "C" void moe_route_launcher(int* ids, float* weights, const float* logits, int tokens,
                                    int n_experts, int top_k, int config, hipStream_t stream) {
-    (void)config;
+    const int shared = (config & CONFIG_SHARED_SLOT) ? 1 : 0;
     if (tokens <= 0) return;
-    if (n_experts <= 0 || n_experts > 512 || top_k <= 0 || top_k > 64 || top_k > n_experts) {
+    if (n_experts <= 0 || n_experts > 512 - shared || top_k <= 0 || top_k > 64 - shared ||
+        top_k > n_experts) {
         caa::set_status(CAA_UNSUPPORTED_SHAPE);
         return;
     }
@@ -436,9 +449,11 @@ extern "C" void moe_route_launcher(int* ids, float* weights, const float* logits
     }
     const int blocks = (tokens + 3) / 4;
     if (n_experts <= 256) {
-        moe_route_kernel<4><<<blocks, 256, 0, stream>>>(logits, ids, weights, tokens, n_experts, top_k);
+        moe_route_kernel<4><<<blocks, 256, 0, stream>>>(logits, ids, weights, tokens, n_experts, top_k,
+                                                        shared);
     } else {
-        moe_route_kernel<8><<<blocks, 256, 0, stream>>>(logits, ids, weights, tokens, n_experts, top_k);
+        moe_route_kernel<8><<<blocks, 256, 0, stream>>>(logits, ids, weights, tokens, n_experts, top_k,
+                                                        shared);
     }
 }
 
@@ -512,8 +527,11 @@ extern "C" void moe_route_sort_launcher(int* ids, float* weights, int* sorted_pa
                                         int* expert_offsets, int* chunk_scratch, const float* logits,
                                         int tokens, int n_experts, int top_k, int config,
                                         hipStream_t stream) {
+    const int shared = (config & CONFIG_SHARED_SLOT) ? 1 : 0;
+    config &= ~CONFIG_SHARED_SLOT;
     if (tokens <= 0) return;
-    if (n_experts <= 0 || n_experts > 512 || top_k <= 0 || top_k > 64 || top_k > n_experts) {
+    if (n_experts <= 0 || n_experts > 512 - shared || top_k <= 0 || top_k > 64 - shared ||
+        top_k > n_experts) {
         caa::set_status(CAA_UNSUPPORTED_SHAPE);
         return;
     }
@@ -521,17 +539,19 @@ extern "C" void moe_route_sort_launcher(int* ids, float* weights, int* sorted_pa
         caa::set_status(CAA_BAD_ARGUMENT);
         return;
     }
-    if ((long)tokens * top_k <= 1024 && config != 1) {
+    if ((long)tokens * (top_k + shared) <= 1024 && config != 1) {
         if (n_experts <= 256) {
             moe_route_sort_small_kernel<4><<<1, 1024, 0, stream>>>(
-                logits, ids, weights, sorted_pairs, pair_pos, expert_offsets, tokens, n_experts, top_k);
+                logits, ids, weights, sorted_pairs, pair_pos, expert_offsets, tokens, n_experts, top_k,
+                shared);
         } else {
             moe_route_sort_small_kernel<8><<<1, 1024, 0, stream>>>(
-                logits, ids, weights, sorted_pairs, pair_pos, expert_offsets, tokens, n_experts, top_k);
+                logits, ids, weights, sorted_pairs, pair_pos, expert_offsets, tokens, n_experts, top_k,
+                shared);
         }
         return;
     }
-    moe_route_launcher(ids, weights, logits, tokens, n_experts, top_k, 0, stream);
-    moe_sort_launcher(sorted_pairs, pair_pos, expert_offsets, chunk_scratch, ids, tokens, n_experts,
-                      top_k, 0, stream);
+    moe_route_launcher(ids, weights, logits, tokens, n_experts, top_k, shared ? CONFIG_SHARED_SLOT : 0, stream);
+    moe_sort_launcher(sorted_pairs, pair_pos, expert_offsets, chunk_scratch, ids, tokens,
+                      n_experts + shared, top_k + shared, 0, stream);
 }

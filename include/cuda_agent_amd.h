@@ -173,7 +173,10 @@ void topk_select_launcher(int* idx_out, const float* scores, const int* lengths,
 
 /* ids [tokens, top_k] int32: the top_k largest logits of each token, descending, ties to the
  * lower expert id; weights [tokens, top_k] fp32: sigmoid(logit) normalised over the top_k.
- * logits [tokens, n_experts] fp32. n_experts <= 512, top_k <= 64. */
+ * logits [tokens, n_experts] fp32. n_experts <= 512, top_k <= 64.
+ * config bit 64 (also understood by moe_route_sort_launcher): every token gets one more slot after
+ * its top_k, expert number n_experts with weight 1 (a shared expert stored behind the routed ones);
+ * ids and weights are then [tokens, top_k + 1] and the sort covers n_experts + 1 experts. */
 void moe_route_launcher(int* ids, float* weights, const float* logits, int tokens, int n_experts,
                         int top_k, int config, hipStream_t stream);
 
@@ -289,6 +292,19 @@ void moe_fp8_shared_launcher(void* out, const void* x, const float* logits, cons
                              const float* sw2_s, void* workspace, size_t workspace_bytes, int tokens,
                              int hidden, int inter, int shared_inter, int n_experts, int top_k,
                              int out_dtype, int config, hipStream_t stream);
+
+/* The same layer with the shared expert stored as expert number n_experts behind the routed ones
+ * (w13_q [n_experts + 1, 2*inter, hidden], w13_s, w2_q, w2_s likewise; same inter): every token
+ * takes it as one more slot with weight 1, so it runs inside the routed experts' launches rather
+ * than as launches of its own that fill a fraction of the chip. Same sum as above. logits
+ * [tokens, n_experts]. workspace: moe_fp8_workspace_bytes(tokens, hidden, inter, n_experts + 1,
+ * top_k + 1) bytes, with the layout of that shape (rows of ids/weights have top_k + 1 entries, the
+ * last one the shared expert). n_experts <= 511, top_k <= 63; config as moe_fp8_launcher. */
+void moe_fp8_fused_shared_launcher(void* out, const void* x, const float* logits, const void* w13_q,
+                                   const float* w13_s, const void* w2_q, const float* w2_s,
+                                   void* workspace, size_t workspace_bytes, int tokens, int hidden,
+                                   int inter, int n_experts, int top_k, int out_dtype, int config,
+                                   hipStream_t stream);
 
 #ifdef __cplusplus
 }

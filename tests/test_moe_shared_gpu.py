@@ -75,3 +75,45 @@ def test_rejects_bad_arguments(capi, dev):
     with pytest.raises(capi.LaunchRejected):          # the routed layer's workspace is not enough
         capi.moe_fp8_shared_launch(out, *dts, small, top_k=2)
     torch.cuda.synchronize()
+
+
+# ---- the shared expert stored as one more expert behind the routed ones ---------------------------
+
+def run_fused(capi, dts, top_k, config=0, dtype=torch.float32):
+    x, logits, w13_q, w13_s, w2_q, w2_s, sw13_q, sw13_s, sw2_q, sw2_s = dts
+    stacked = [torch.cat([a, b[None]]) for a, b in ((w13_q, sw13_q), (w13_s, sw13_s), (w2_q, sw2_q), (w2_s, sw2_s))]
+    T, H = x.shape
+    E, I2, _ = w13_q.shape
+    ws = torch.empty(capi.moe_workspace_bytes(T, H, I2 // 2, E + 1, top_k + 1), dtype=torch.uint8, device=x.device)
+    out = torch.full((T, H), float('nan'), dtype=dtype, device=x.device)
+    capi.moe_fp8_fused_shared_launch(out, x, logits, *stacked, ws, top_k=top_k, config=config)
+    torch.cuda.synchronize()
+    return out, capi.moe_workspace_views(ws, T, H, I2 // 2, E + 1, top_k + 1)
+
+
+@pytest.mark.parametrize('config', [16, 4, 0])
+@pytest.mark.parametrize('shape', [(64, 512, 256, 16, 4), (300, 256, 128, 8, 2), (1, 256, 128, 4, 1),
+                                   (1100, 512, 256, 5, 2), (33, 768, 384, 40, 8), (128, 512, 256, 256, 7)])
+def test_shared_expert_inside_the_routed_launch(capi, dev, shape, config):
+    T, H, I, E, k = shape
+    x, logits, w, sw, dts = make_case(dev, T, H, I, I, E, 4000 + T)
+    fused, views = run_fused(capi, dts, k, config)
+    assert torch.isfinite(fused).all()
+    # routing: the first k slots are the plain router's, the last one is the shared expert with weight 1
+    want_ids, want_w = moe.route(logits, k)
+    ids = views['ids'].cpu().reshape(T, k + 1)
+    wts = views['weights'].cpu().reshape(T, k + 1)
+    assert torch.equal(ids[:, :k], want_ids) and (ids[:, k] == E).all() and (wts[:, k] == 1).all()
+    torch.testing.assert_close(wts[:, :k], want_w, rtol=1e-6, atol=1e-7)
+    sp, pos, off = moe.sort_pairs(ids, E + 1)
+    assert torch.equal(views['sorted_pairs'].cpu(), sp) and torch.equal(views['expert_offsets'].cpu(), off)
+    if config:
+        # same GEMM form in both layers: the same tiles are computed and summed in the same order
+        assert torch.equal(fused, run_shared(capi, dts, k, config, torch.float32))
+    ref = moe.moe_forward_shared(x, logits, *w, *sw, top_k=k, out_dtype=torch.float32)
+    rms = ref.double().pow(2).mean().sqrt()
+    diff = (fused.cpu() - ref).double().abs()
+    assert (diff.pow(2).mean().sqrt() / rms).item() <= 5e-3
+    assert (diff > TOL * rms).double().mean().item() <= 1e-3
+    assert (diff.max() / rms).item() <= 0.15
+    assert torch.equal(run_fused(capi, dts, k, config, torch.bfloat16)[0], fused.bfloat16())
