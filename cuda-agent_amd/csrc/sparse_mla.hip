@@ -599,6 +599,18 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
         const int i = tid + 512 * j;
         raw_key[j] = i < n_rows ? idx[(size_t)b * topk + row_begin + i] : -1;
     }
+    // Q^T operand of this wavefront's share of d: local step l is k-step 4*(l/2) + 2*dh + l%2,
+    // i.e. the two wavefronts of a pair alternate 32-element slices of d. The wait for Q also
+    // waits for the two tiles issued above (loads return in order), which the loop needs anyway.
+    // (requested here, behind the indices: Q does not depend on them, so its latency overlaps theirs)
+    bf16x8 qreg[HALF_K_STEPS];
+    {
+        const __bf16* qrow = q + ((size_t)b * n_heads + head0 + (lane & 31)) * D_QK + 8 * half + 32 * dh;
+#pragma unroll
+        for (int l = 0; l < HALF_K_STEPS; ++l) {
+            qreg[l] = *reinterpret_cast<const bf16x8*>(qrow + 64 * (l >> 1) + 16 * (l & 1));
+        }
+    }
     if (kva.block_table != nullptr) {
 #pragma unroll
         for (int j = 0; j < MAX_SPLIT_ROWS / 512; ++j)
@@ -643,17 +655,6 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
     }
     PHASE_MARK(9);  // first gather issue
 
-    // Q^T operand of this wavefront's share of d: local step l is k-step 4*(l/2) + 2*dh + l%2,
-    // i.e. the two wavefronts of a pair alternate 32-element slices of d. The wait for Q also
-    // waits for the two tiles issued above (loads return in order), which the loop needs anyway.
-    bf16x8 qreg[HALF_K_STEPS];
-    {
-        const __bf16* qrow = q + ((size_t)b * n_heads + head0 + (lane & 31)) * D_QK + 8 * half + 32 * dh;
-#pragma unroll
-        for (int l = 0; l < HALF_K_STEPS; ++l) {
-            qreg[l] = *reinterpret_cast<const bf16x8*>(qrow + 64 * (l >> 1) + 16 * (l & 1));
-        }
-    }
 #pragma unroll
     for (int ks = 0; ks < HALF_K_STEPS; ++ks) asm volatile("" : "+v"(qreg[ks]));
     PHASE_MARK(8);  // wait for Q
