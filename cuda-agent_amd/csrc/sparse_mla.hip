@@ -492,7 +492,7 @@ __global__ __launch_bounds__(64 * NW) void sparse_mla_split_kernel(
 // Measured per wavefront and tile (core clock cycles, 16-tile splits): gather issue 2 000 (the
 // memory pipeline accepts one 1 KB load of a wavefront per 150-300 cycles, whatever the
 // addresses), QK^T 950-1 200, softmax + rescale 1 750-1 950, PV 650-900, barriers 500-2 800;
-// the prologue (indices, Q, first tiles) is 10 us and the epilogue (262 KB of partials) 5 us.
+// the prologue (indices, Q, first tiles) is 10 us and the epilogue (131 KB of fp16 partials) 3 us.
 // ---------------------------------------------------------------------------------------------
 // Phase timing build (-DMLA_PHASE_TIMING): every wavefront of workgroup (0,0,0) adds up the core
 // clock cycles it spends in each phase of the loop and leaves them in g_phase_cycles.
@@ -561,14 +561,15 @@ __device__ __forceinline__ void gather_issue(uint4* tile, const char* kv_b, uint
 // grid: x = split, y = request, z = group of 128 heads; 512 lanes
 __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ kv, const int* __restrict__ idx,
-    float* __restrict__ o_part, float* __restrict__ lse_part, int n_heads, int n_kv_rows, int topk,
-    int rows_per_split, float scale_log2, KvAddressing kva) {
+    _Float16* __restrict__ o_part, float* __restrict__ lse_part, float* __restrict__ scale_part,
+    int n_heads, int n_kv_rows, int topk, int rows_per_split, float scale_log2, KvAddressing kva) {
     typedef const __attribute__((address_space(3))) uintx4* lds_x4;
     typedef shortx4 __attribute__((address_space(3)))* lds_s4;
     __shared__ uint4 tiles[3 * TILE_CHUNKS];  // ring of three resident tiles
     __shared__ floatx4 s_xchg[8][4 * 64];     // partial scores of every wavefront, 4 KB each
     __shared__ int s_idx[MAX_SPLIT_ROWS];
     __shared__ uint32_t s_gather_tab[GATHER_TAB];
+    __shared__ float s_head_max[8][32];  // epilogue: largest |O^T| of every head in a wavefront's half
     __shared__ int s_first_masked_tile;
 
     PHASE_TIMING_BEGIN();
@@ -827,17 +828,34 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
     }
 
     // epilogue: normalise; O^T half -> LDS (64 dv at a time, region private to the wavefront)
-    // -> 256-byte row segments of the partial output
+    // -> 128-byte row segments of the partial output. The partial is stored as fp16 of
+    // O / 2^e with 2^e the power of two above the head's largest magnitude (kept next to the
+    // log-sum-exp): half the bytes of fp32 for the split kernel to write and the merge to read, and
+    // an error of at most 2^-12 of that magnitude.
     const float l_total = st.l + __shfl_xor(st.l, 32);
     const float inv_l = l_total > 0.f ? 1.f / l_total : 0.f;
     const size_t part0 = ((size_t)b * n_splits + split) * n_heads + head0;
+    float amax = 0.f;
+#pragma unroll
+    for (int t = 0; t < 8; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(acc[t][i]));
+    amax = fmaxf(amax, __shfl_xor(amax, 32));
+    if (half == 0) s_head_max[wave][lane] = amax;
     if (dh == 0 && half == 0) {
         lse_part[part0 + lane] = l_total > 0.f ? st.m + __builtin_amdgcn_logf(l_total) : -INFINITY;
     }
     __syncthreads();
+    // exponent field of the bound + 1: 2^e > |O| for every element of the head (1 if the head is 0)
+    const float bound = fmaxf(s_head_max[wave][lane & 31], s_head_max[wave ^ 1][lane & 31]) * inv_l;
+    uint32_t e_bits = ((__float_as_uint(bound) >> 23) & 255u) + 1u;
+    e_bits = bound > 0.f ? (e_bits > 253u ? 253u : e_bits) : 127u;
+    const float inv_scale = __uint_as_float((254u - e_bits) << 23) * inv_l;
+    if (dh == 0 && half == 0) scale_part[part0 + lane] = __uint_as_float(e_bits << 23);
     constexpr int STAGE_STRIDE = 64 + 4;
     float* stage = reinterpret_cast<float*>(tiles + (wave >> 2) * TILE_CHUNKS) + (wave & 3) * (32 * STAGE_STRIDE);
-    float* o_rows = o_part + part0 * D_V + 256 * dh;
+    _Float16* o_rows = o_part + part0 * D_V + 256 * dh;
+    typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
 #pragma unroll
     for (int ps = 0; ps < 4; ++ps) {
 #pragma unroll
@@ -845,8 +863,8 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
             const floatx16 a = acc[2 * ps + tt];
 #pragma unroll
             for (int qd = 0; qd < 4; ++qd) {
-                floatx4 v = {a[4 * qd] * inv_l, a[4 * qd + 1] * inv_l, a[4 * qd + 2] * inv_l,
-                             a[4 * qd + 3] * inv_l};
+                floatx4 v = {a[4 * qd] * inv_scale, a[4 * qd + 1] * inv_scale, a[4 * qd + 2] * inv_scale,
+                             a[4 * qd + 3] * inv_scale};
                 *reinterpret_cast<floatx4*>(stage + (lane & 31) * STAGE_STRIDE + 32 * tt + 8 * qd +
                                             4 * half) = v;
             }
@@ -855,7 +873,8 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
         for (int it = 0; it < 8; ++it) {
             const int r = 4 * it + (lane >> 4);
             const floatx4 v = *reinterpret_cast<const floatx4*>(stage + r * STAGE_STRIDE + 4 * (lane & 15));
-            *reinterpret_cast<floatx4*>(o_rows + (size_t)r * D_V + 64 * ps + 4 * (lane & 15)) = v;
+            const halfx4 h = {(_Float16)v.x, (_Float16)v.y, (_Float16)v.z, (_Float16)v.w};
+            *reinterpret_cast<halfx4*>(o_rows + (size_t)r * D_V + 64 * ps + 4 * (lane & 15)) = h;
         }
     }
     PHASE_MARK(10);  // epilogue
@@ -863,12 +882,15 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
 }
 
 // out[b, h, :] = sum_s w_s o_part[b, s, h, :],  w_s = exp2(lse_s - max) / sum; one workgroup of
-// 128 lanes per (b, h), 4 output columns per lane.
-template <typename OUT>
-__global__ __launch_bounds__(128) void sparse_mla_merge_kernel(const float* __restrict__ o_part,
+// 128 lanes per (b, h), 4 output columns per lane. PART is the type the split kernel stored:
+// float, or fp16 of O / scale with the per-head scale in scale_part.
+template <typename OUT, typename PART>
+__global__ __launch_bounds__(128) void sparse_mla_merge_kernel(const PART* __restrict__ o_part,
                                                                const float* __restrict__ lse_part,
+                                                               const float* __restrict__ scale_part,
                                                                OUT* __restrict__ out, int n_heads,
                                                                int n_splits) {
+    typedef PART partx4 __attribute__((ext_vector_type(4)));
     const int h = blockIdx.x;
     const int b = blockIdx.y;
     const size_t base = (size_t)b * n_splits * n_heads + h;
@@ -880,8 +902,10 @@ __global__ __launch_bounds__(128) void sparse_mla_merge_kernel(const float* __re
         for (int s = 0; s < n_splits; ++s) {
             const float w = __builtin_amdgcn_exp2f(lse_part[base + (size_t)s * n_heads] - mx);
             if (w > 0.f) {
-                const floatx4 v = *reinterpret_cast<const floatx4*>(
+                const partx4 p = *reinterpret_cast<const partx4*>(
                     o_part + (base + (size_t)s * n_heads) * D_V + threadIdx.x * 4);
+                floatx4 v = {(float)p.x, (float)p.y, (float)p.z, (float)p.w};
+                if constexpr (sizeof(PART) == 2) v *= scale_part[base + (size_t)s * n_heads];
                 o += v * w;
                 wsum += w;
             }
@@ -924,7 +948,8 @@ extern "C" int sparse_mla_decode_num_splits(int batch, int n_heads, int topk, in
 // bytes of scratch sparse_mla_decode_launcher needs for these sizes
 extern "C" size_t sparse_mla_decode_workspace_bytes(int batch, int n_heads, int topk, int config) {
     const int splits = sparse_mla_decode_num_splits(batch, n_heads, topk, config);
-    return (size_t)batch * splits * n_heads * (D_V + 1) * sizeof(float);
+    // partial outputs (sized for fp32), log-sum-exp and scale of every (request, split, head)
+    return (size_t)batch * splits * n_heads * (D_V + 2) * sizeof(float);
 }
 
 namespace {
@@ -965,10 +990,13 @@ void launch_sparse_mla(void* out, const void* q, const void* kv, const int* idx,
     const int rows_per_split = ((tiles + splits - 1) / splits) * TILE_ROWS;
     float* o_part = static_cast<float*>(workspace);
     float* lse_part = o_part + (size_t)batch * splits * n_heads * D_V;
+    float* scale_part = lse_part + (size_t)batch * splits * n_heads;
     const float scale_log2 = sm_scale * 1.4426950408889634f;
     const __bf16* qb = static_cast<const __bf16*>(q);
     const __bf16* kvb = static_cast<const __bf16*>(kv);
     const dim3 grid(splits, batch, head_groups);
+    const dim3 merge_grid(n_heads, batch);
+    bool half_parts = false;
     if (n_heads == 32) {
         sparse_mla_split_kernel<1><<<grid, 64, 0, stream>>>(qb, kvb, idx, o_part, lse_part, n_heads,
                                                             n_kv_rows, topk, rows_per_split,
@@ -982,16 +1010,26 @@ void launch_sparse_mla(void* out, const void* q, const void* kv, const int* idx,
                                                              n_kv_rows, topk, rows_per_split,
                                                              scale_log2, kva);
     } else {
-        sparse_mla_split8_kernel<<<grid, 512, 0, stream>>>(qb, kvb, idx, o_part, lse_part, n_heads,
-                                                           n_kv_rows, topk, rows_per_split,
-                                                           scale_log2, kva);
+        half_parts = true;  // this kernel stores its partials as scaled fp16
+        sparse_mla_split8_kernel<<<grid, 512, 0, stream>>>(
+            qb, kvb, idx, reinterpret_cast<_Float16*>(o_part), lse_part, scale_part, n_heads, n_kv_rows,
+            topk, rows_per_split, scale_log2, kva);
     }
-    if (out_dtype == 0) {
-        sparse_mla_merge_kernel<__bf16><<<dim3(n_heads, batch), 128, 0, stream>>>(
-            o_part, lse_part, static_cast<__bf16*>(out), n_heads, splits);
+    if (half_parts) {
+        const _Float16* parts = reinterpret_cast<const _Float16*>(o_part);
+        if (out_dtype == 0) {
+            sparse_mla_merge_kernel<__bf16, _Float16><<<merge_grid, 128, 0, stream>>>(
+                parts, lse_part, scale_part, static_cast<__bf16*>(out), n_heads, splits);
+        } else {
+            sparse_mla_merge_kernel<float, _Float16><<<merge_grid, 128, 0, stream>>>(
+                parts, lse_part, scale_part, static_cast<float*>(out), n_heads, splits);
+        }
+    } else if (out_dtype == 0) {
+        sparse_mla_merge_kernel<__bf16, float><<<merge_grid, 128, 0, stream>>>(
+            o_part, lse_part, nullptr, static_cast<__bf16*>(out), n_heads, splits);
     } else {
-        sparse_mla_merge_kernel<float><<<dim3(n_heads, batch), 128, 0, stream>>>(
-            o_part, lse_part, static_cast<float*>(out), n_heads, splits);
+        sparse_mla_merge_kernel<float, float><<<merge_grid, 128, 0, stream>>>(
+            o_part, lse_part, nullptr, static_cast<float*>(out), n_heads, splits);
     }
 }
 
