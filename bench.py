@@ -120,6 +120,38 @@ def bench_gdn(torch, capi, dev, steps, warmup, cpu_baseline):
     return res
 
 
+def bench_gdn_fused_norm(torch, capi, dev, steps, warmup, cpu_baseline):
+    """configs[1] sizes through the launcher that does the pre-step, the recurrence and the gated RMS
+    normalisation of the read-out: the gate z is read (bf16) and the output is bf16 instead of fp32."""
+    from oracle import gdn
+    B, Hv, Hqk = 256, 32, 16
+    gen = torch.Generator().manual_seed(20261)
+    host = gdn.gdn_make_raw_inputs(B, Hv, Hqk, qkv_dtype=torch.bfloat16, generator=gen)
+    hz = (torch.randn(B, Hv, 128, generator=gen) * 2).bfloat16()
+    hw = (1.0 + 0.1 * torch.randn(128, generator=gen)).bfloat16()
+    q, k, v, a, b, a_log, dt_bias, state0 = (t.to(dev) for t in host)
+    z, norm_w = hz.to(dev), hw.to(dev)
+    sets = [(torch.empty(B, Hv, 128, dtype=torch.bfloat16, device=dev), state0.clone()) for _ in range(3)]
+    sec = timed_launches(
+        torch, lambda i: capi.gdn_decode_fused_norm_launch(*sets[i % 3], q, k, v, a, b, a_log, dt_bias, z, norm_w),
+        steps, warmup)
+    work = 2 * B * Hv * 128 * 128 * 4 + 2 * B * Hqk * 128 * 2 + 3 * B * Hv * 128 * 2 + 2 * B * Hv * 4 + 2 * Hv * 4 + 256
+    res = dict(
+        workload="configs[1] sizes with the pre-step and the gated RMS normalisation of the read-out fused "
+                 "(bf16 gate in, bf16 output), seed 20261",
+        value=work / sec / 1e9, unit="GB/s", ms_per_step=sec * 1e3, dtype="f32", kernel="gdn_decode_kernel<fused,norm>",
+        roofline=dict(bound="hbm", achieved=work / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
+                      frac=work / sec / 1e9 / HBM_PEAK_GBS, traffic=None),
+        algorithmic_bytes=work)
+    if cpu_baseline:
+        cores = len(os.sched_getaffinity(0))
+        torch.set_num_threads(cores)
+        csec = cpu_time(lambda: gdn.gdn_decode_fused_norm_step(*host, hz, hw))
+        res['cpu_baseline'] = dict(value=work / csec / 1e9, unit="GB/s", cores=cores, kind="port",
+                                   sample="the full step (eager PyTorch oracle, state in place)")
+    return res
+
+
 def bench_gdn_fused(torch, capi, dev, steps, warmup, cpu_baseline):
     """configs[1] sizes through the launcher that also does the caller's pre-step (L2 normalisation of
     q and k, decay and write gates): same bytes, the gate inputs a, b take the place of g, beta."""
@@ -430,7 +462,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=20)
     ap.add_argument('--warmup', type=int, default=5)
-    ap.add_argument('--workloads', default='gdn,gdn_fused,conv1d,moe_decode,router_decode,topk_select,mla,mla_paged,moe_prefill,router_prefill')
+    ap.add_argument('--workloads', default='gdn,gdn_fused,gdn_fused_norm,conv1d,moe_decode,router_decode,topk_select,mla,mla_paged,moe_prefill,router_prefill')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run 3 plain device copies of 536 870 912 bytes (a kernel of known traffic, '
@@ -463,6 +495,8 @@ def main():
             results[name] = bench_gdn(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'gdn_fused':
             results[name] = bench_gdn_fused(torch, capi, dev, args.steps, args.warmup, cpu)
+        elif name == 'gdn_fused_norm':
+            results[name] = bench_gdn_fused_norm(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'conv1d':
             results[name] = bench_conv1d(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name in ('router_decode', 'router_prefill'):

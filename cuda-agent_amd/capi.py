@@ -22,6 +22,8 @@ SIGNATURES = {
                                    c_int, c_int, _P]),
     'gdn_decode_fused_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int,
                                          c_int, c_int, c_int, _P]),
+    'gdn_decode_fused_norm_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_float, c_int, c_int,
+                                              c_int, c_int, c_int, c_int, c_int, _P]),
     'causal_conv1d_update_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int,
                                              c_int, c_int, c_int, _P]),
     'sparse_mla_decode_launcher': (None, [_P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int,
@@ -162,6 +164,32 @@ def gdn_decode_fused_launch(o, state, q, k, v, a, b, a_log, dt_bias, config=0, s
                                         0 if q.dtype == torch.float32 else 1, config, _stream(stream))
     check_status('gdn_decode_fused_launcher')
     return o, state
+
+
+def gdn_decode_fused_norm_launch(out, state, q, k, v, a, b, a_log, dt_bias, z, norm_w, eps=1e-6, config=0,
+                                 stream=None):
+    """The fused step plus the gated RMS normalisation of its read-out: out [B,Hv,128] (dtype of q/k/v) =
+    norm_w * o * rsqrt(mean(o^2) + eps) * silu(z); state updated in place."""
+    import torch
+    _device_contiguous(out=out, state=state, q=q, k=k, v=v, a=a, b=b, a_log=a_log, dt_bias=dt_bias, z=z,
+                       norm_w=norm_w)
+    B, Hv, dk, dv = state.shape
+    Hqk = q.shape[1]
+    _require(state.dtype == torch.float32, 'gdn_decode: state must be fp32')
+    _require(q.dtype == k.dtype == v.dtype == z.dtype == norm_w.dtype == out.dtype
+             and q.dtype in (torch.float32, torch.bfloat16), 'gdn_decode: q, k, v, z, norm_w, out of one type')
+    _require(all(t.dtype == torch.float32 for t in (a, b, a_log, dt_bias)), 'gdn_decode: gate tensors must be fp32')
+    _require(tuple(q.shape) == tuple(k.shape) == (B, Hqk, dk) and tuple(v.shape) == (B, Hv, dv), 'gdn_decode: q/k/v')
+    _require(tuple(z.shape) == tuple(out.shape) == (B, Hv, dv) and tuple(norm_w.shape) == (dv,),
+             'gdn_decode: z/out [B,Hv,dv], norm_w [dv]')
+    _require(tuple(a.shape) == tuple(b.shape) == (B, Hv) and tuple(a_log.shape) == tuple(dt_bias.shape) == (Hv,),
+             'gdn_decode: gate shapes')
+    library().gdn_decode_fused_norm_launcher(
+        _ptr(out), _ptr(state), _ptr(q), _ptr(k), _ptr(v), _ptr(a), _ptr(b), _ptr(a_log), _ptr(dt_bias), _ptr(z),
+        _ptr(norm_w), float(eps), B, Hv, Hqk, dk, dv, 0 if q.dtype == torch.float32 else 1, config,
+        _stream(stream))
+    check_status('gdn_decode_fused_norm_launcher')
+    return out, state
 
 
 def causal_conv1d_update_launch(q_out, k_out, v_out, conv_state, x, weight, bias=None, activation='silu',

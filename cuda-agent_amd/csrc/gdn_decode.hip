@@ -36,6 +36,8 @@ constexpr int DV = 128;
 
 __device__ __forceinline__ float to_f32(float x) { return x; }
 __device__ __forceinline__ float to_f32(__hip_bfloat16 x) { return __bfloat162float(x); }
+__device__ __forceinline__ void from_f32(float& d, float x) { d = x; }
+__device__ __forceinline__ void from_f32(__hip_bfloat16& d, float x) { d = __float2bfloat16(x); }
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
@@ -60,12 +62,19 @@ __device__ __forceinline__ void store_state(float* p, float4 x, bool nt) {
 // FUSED: q and k arrive unnormalised and are scaled by rsqrt(sum x^2 + 1e-6) here (the factors are
 // applied to the reductions, not to the 128 values); `g` and `beta` are then the per-request
 // gate inputs a and b, and g = exp(-exp(a_log[h]) * softplus(a + dt_bias[h])), beta = sigmoid(b).
-template <typename T, int COLS, int THREADS, int NT, bool FUSED = false>
+//
+// NORM (needs COLS == DV, one workgroup per head): the layer's gated RMS normalisation of the read-out
+// is applied before it is stored: out = norm_w * o * rsqrt(mean(o^2) + eps) * silu(z), written in
+// the storage type of q/k/v to o_norm; the fp32 o is not written.
+template <typename T, int COLS, int THREADS, int NT, bool FUSED = false, bool NORM = false>
 __global__ __launch_bounds__(THREADS) void gdn_decode_kernel(
     float* __restrict__ o, float* __restrict__ state, const T* __restrict__ q,
     const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ g,
     const float* __restrict__ beta, int n_v_heads, int n_qk_heads, float scale,
-    const float* __restrict__ a_log = nullptr, const float* __restrict__ dt_bias = nullptr) {
+    const float* __restrict__ a_log = nullptr, const float* __restrict__ dt_bias = nullptr,
+    const T* __restrict__ z = nullptr, const T* __restrict__ norm_w = nullptr, float norm_eps = 0.f,
+    T* __restrict__ o_norm = nullptr) {
+    static_assert(!NORM || COLS == DV, "the normalisation needs a head's whole read-out in one workgroup");
     constexpr int WAVES = THREADS / 64;
     constexpr int CG = COLS / 4;            // float4 column groups per row segment
     constexpr int RPP = THREADS / CG;       // rows covered by one pass of the workgroup
@@ -127,6 +136,14 @@ __global__ __launch_bounds__(THREADS) void gdn_decode_kernel(
 #pragma unroll
     for (int m = 0; m < NP; ++m) {
         s[m] = load_state(S + (size_t)(r0 + m * RPP) * DV, NT == 1 || NT == 2);
+    }
+    // NORM: the lanes that will hold the read-out (r0 == 0) fetch their gate and weight values now
+    float4 zj = make_float4(0.f, 0.f, 0.f, 0.f), wj = zj;
+    if (NORM && r0 == 0) {
+        const T* zh = z + (size_t)unit * DV + cg * 4;
+        const T* wh = norm_w + cg * 4;
+        zj = make_float4(to_f32(zh[0]), to_f32(zh[1]), to_f32(zh[2]), to_f32(zh[3]));
+        wj = make_float4(to_f32(wh[0]), to_f32(wh[1]), to_f32(wh[2]), to_f32(wh[3]));
     }
 
     float kq_part = 0.f;
@@ -223,12 +240,12 @@ __global__ __launch_bounds__(THREADS) void gdn_decode_kernel(
     d.z = bh * (vj.z - gh * a.z);
     d.w = bh * (vj.w - gh * a.w);
 
-    if (r0 == 0) {
-        float4 ov;
-        ov.x = scale * (gh * c.x + kq * d.x);
-        ov.y = scale * (gh * c.y + kq * d.y);
-        ov.z = scale * (gh * c.z + kq * d.z);
-        ov.w = scale * (gh * c.w + kq * d.w);
+    float4 ov;
+    ov.x = scale * (gh * c.x + kq * d.x);
+    ov.y = scale * (gh * c.y + kq * d.y);
+    ov.z = scale * (gh * c.z + kq * d.z);
+    ov.w = scale * (gh * c.w + kq * d.w);
+    if (!NORM && r0 == 0) {
         *reinterpret_cast<float4*>(o + (size_t)unit * DV + tile * COLS + cg * 4) = ov;
     }
 
@@ -240,6 +257,20 @@ __global__ __launch_bounds__(THREADS) void gdn_decode_kernel(
         n.z = gh * s[m].z + kr[m] * d.z;
         n.w = gh * s[m].w + kr[m] * d.w;
         store_state(S + (size_t)(r0 + m * RPP) * DV, n, NT == 1 || NT == 3);
+    }
+
+    if (NORM && r0 == 0) {
+        // lanes 0..CG-1 (CG == 32: the lower half of wavefront 0) hold the head's 128 values
+        float ss = ov.x * ov.x + ov.y * ov.y + ov.z * ov.z + ov.w * ov.w;
+#pragma unroll
+        for (int off = CG / 2; off >= 1; off >>= 1) ss += __shfl_xor(ss, off);
+        const float rinv = rsqrtf(ss * (1.f / DV) + norm_eps);
+        auto gated = [&](float x, float w, float zz) { return w * (x * rinv) * (zz / (1.f + __expf(-zz))); };
+        T* dst = o_norm + (size_t)unit * DV + cg * 4;
+        const float r[4] = {gated(ov.x, wj.x, zj.x), gated(ov.y, wj.y, zj.y), gated(ov.z, wj.z, zj.z),
+                            gated(ov.w, wj.w, zj.w)};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) from_f32(dst[i], r[i]);
     }
 }
 
@@ -352,5 +383,46 @@ extern "C" void gdn_decode_fused_launcher(float* o, float* state, const void* q,
     } else {
         launch<__hip_bfloat16>(o, state, q, k, v, a, b, a_log, dt_bias, batch, n_v_heads, n_qk_heads, config,
                                stream);
+    }
+}
+
+
+// gdn_decode_fused_launcher followed by the layer's gated RMS normalisation of the read-out, in the
+// same kernel: out [batch, n_v_heads, 128] in the storage type of q/k/v (qkv_dtype) =
+//   norm_w * o * rsqrt(mean_j(o_j^2) + eps) * silu(z),   o the step's fp32 read-out (not stored),
+// z [batch, n_v_heads, 128] the output gate and norm_w [128] the norm's weight, both of that type.
+// config is accepted for the launcher pattern and has one value (one workgroup of 1024 lanes per head).
+extern "C" void gdn_decode_fused_norm_launcher(void* out, float* state, const void* q, const void* k,
+                                               const void* v, const float* a, const float* b,
+                                               const float* a_log, const float* dt_bias,
+                                               const void* z, const void* norm_w, float eps, int batch,
+                                               int n_v_heads, int n_qk_heads, int dk, int dv,
+                                               int qkv_dtype, int config, hipStream_t stream) {
+    (void)config;
+    if (batch <= 0 || n_v_heads <= 0) return;
+    if (!gdn_shape_ok(batch, n_v_heads, n_qk_heads, dk, dv, qkv_dtype)) {
+        caa::set_status(CAA_UNSUPPORTED_SHAPE);
+        return;
+    }
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(state);
+    if (!out || !state || !q || !k || !v || !a || !b || !a_log || !dt_bias || !z || !norm_w ||
+        (bits & 15u) != 0) {
+        caa::set_status(CAA_BAD_ARGUMENT);
+        return;
+    }
+    const int units = batch * n_v_heads;
+    const float scale = 0.08838834764831845f;  // 128^-1/2
+    if (qkv_dtype == 0) {
+        typedef float T;
+        gdn_decode_kernel<T, 128, 1024, 1, true, true><<<units, 1024, 0, stream>>>(
+            nullptr, state, static_cast<const T*>(q), static_cast<const T*>(k), static_cast<const T*>(v), a,
+            b, n_v_heads, n_qk_heads, scale, a_log, dt_bias, static_cast<const T*>(z),
+            static_cast<const T*>(norm_w), eps, static_cast<T*>(out));
+    } else {
+        typedef __hip_bfloat16 T;
+        gdn_decode_kernel<T, 128, 1024, 1, true, true><<<units, 1024, 0, stream>>>(
+            nullptr, state, static_cast<const T*>(q), static_cast<const T*>(k), static_cast<const T*>(v), a,
+            b, n_v_heads, n_qk_heads, scale, a_log, dt_bias, static_cast<const T*>(z),
+            static_cast<const T*>(norm_w), eps, static_cast<T*>(out));
     }
 }

@@ -80,6 +80,20 @@ void gdn_decode_fused_launcher(float* o, float* state, const void* q, const void
                                const float* dt_bias, int batch, int n_v_heads, int n_qk_heads,
                                int dk, int dv, int qkv_dtype, int config, hipStream_t stream);
 
+/* gdn_decode_fused_launcher with the step after it in the same kernel: the layer's gated RMS
+ * normalisation of the read-out (same launcher pattern; caller-side neighbour):
+ *   out [batch, n_v_heads, 128], in the storage type of q/k/v =
+ *       norm_w * o * rsqrt(mean_j(o_j^2) + eps) * silu(z)
+ *   o the step's fp32 read-out (not stored), z [batch, n_v_heads, 128] the output gate and
+ *   norm_w [128] the norm's weight, both in the storage type of q/k/v.
+ * Everything else as gdn_decode_fused_launcher. config: one value (0). */
+void gdn_decode_fused_norm_launcher(void* out, float* state, const void* q, const void* k,
+                                    const void* v, const float* a, const float* b,
+                                    const float* a_log, const float* dt_bias, const void* z,
+                                    const void* norm_w, float eps, int batch, int n_v_heads,
+                                    int n_qk_heads, int dk, int dv, int qkv_dtype, int config,
+                                    hipStream_t stream);
+
 /* Short causal depthwise convolution, single-token update: the step before the GDN decode step
  * in a Qwen3-Next-style layer (launcher pattern agent_workdir/kernels/axpby.cu:12-20; not one of
  * the benchmark's workloads, the caller-side neighbour of gdn_decode_fused_launcher). Per request

@@ -25,6 +25,11 @@ float64 closed forms, limits (a_log -> -inf gives g = 1), and a second golden fi
 third-party function called with its in-kernel L2 normalisation switched on and the gate computed by
 library calls (tests/golden/make_gdn_golden.py, ``gdn_fused_golden.npz``).
 
+``gated_rmsnorm`` is the step after the recurrence in the same layer (RMS normalisation of the read-out
+over the head dimension, times a weight, times silu of an output gate). Pinned by: the closed form in
+float64, unit-rms of the normalised vector, gate z = 0 gives 0, and a golden fixture from the third-party
+layer's own norm module in fp32 (``gated_rmsnorm_golden.npz``).
+
 ``causal_conv1d_update`` is the step before that one in the same layer (short depthwise causal
 convolution over the q|k|v projection, single token, state shifted in place). Pinned by: scalar
 loops, the library convolution ``F.conv1d(groups=C)`` over the concatenated sequence, the identity
@@ -101,6 +106,21 @@ def gdn_make_raw_inputs(batch, n_v_heads, n_qk_heads, dk=128, dv=128, qkv_dtype=
     dt_bias = 2 * torch.rand(n_v_heads, generator=gen) - 1
     state = 0.02 * torch.randn(batch, n_v_heads, dk, dv, generator=gen)
     return [q.to(qkv_dtype), k.to(qkv_dtype), v.to(qkv_dtype), a, b, a_log, dt_bias, state]
+
+
+def gated_rmsnorm(o, z, weight, eps=1e-6):
+    """weight * o * rsqrt(mean(o^2, -1) + eps) * silu(z) in fp32, rounded once to z's dtype.
+    o [..., d] fp32 read-out, z [..., d] gate, weight [d]."""
+    of = o.float()
+    zf = z.float()
+    y = weight.float() * (of * torch.rsqrt(of.pow(2).mean(dim=-1, keepdim=True) + eps))
+    return (y * (zf * torch.sigmoid(zf))).to(z.dtype)
+
+
+def gdn_decode_fused_norm_step(q_raw, k_raw, v, a, b, a_log, dt_bias, state, z, norm_w, eps=1e-6):
+    """``gdn_decode_fused_step`` followed by ``gated_rmsnorm`` of its read-out. Returns (out, state)."""
+    o, state = gdn_decode_fused_step(q_raw, k_raw, v, a, b, a_log, dt_bias, state)
+    return gated_rmsnorm(o, z, norm_w, eps), state
 
 
 def causal_conv1d_update(x, conv_state, weight, bias=None, activation='silu'):

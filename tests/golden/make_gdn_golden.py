@@ -69,6 +69,19 @@ def main():
     np.savez_compressed(out, **arrays)
     print('wrote', out, out.stat().st_size, 'bytes')
 
+    # the layer's gated RMS norm (fp32 module: no intermediate roundings)
+    from transformers.models.qwen3_next.modeling_qwen3_next import Qwen3NextRMSNormGated
+    gen = torch.Generator().manual_seed(474747)
+    norm = Qwen3NextRMSNormGated(128, eps=1e-6)
+    with torch.no_grad():
+        norm.weight.copy_(1.0 + 0.1 * torch.randn(128, generator=gen))
+        o = torch.randn(6, 128, generator=gen) * torch.exp(torch.randn(6, 1, generator=gen))
+        z = torch.randn(6, 128, generator=gen) * 2
+        y = norm(o, z)
+    out = Path(__file__).with_name('gated_rmsnorm_golden.npz')
+    np.savez_compressed(out, o=o.numpy(), z=z.numpy(), weight=norm.weight.detach().numpy(), y=y.numpy())
+    print('wrote', out, out.stat().st_size, 'bytes')
+
 
 if __name__ == '__main__':
     main()

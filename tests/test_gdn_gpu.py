@@ -196,3 +196,63 @@ def test_fused_full_workload_shape(capi, dev):
     want_o, want_s = gdn.gdn_decode_step(qn.to(dev), kn.to(dev), ins[2].to(dev), g.to(dev), beta.to(dev),
                                          ins[7].to(dev))
     assert gdn.gdn_close(o1, want_o.cpu()) and gdn.gdn_close(s1, want_s.cpu())
+
+
+# ---- the fused step with the gated RMS normalisation of its read-out ------------------------------
+
+def run_fused_norm(capi, dev, ins, z, norm_w, eps=1e-6):
+    q, k, v, a, b, a_log, dt_bias, state = (t.to(dev) for t in ins)
+    s = state.clone()
+    out = torch.full(v.shape, float('nan'), dtype=v.dtype, device=dev)
+    capi.gdn_decode_fused_norm_launch(out, s, q, k, v, a, b, a_log, dt_bias, z.to(dev), norm_w.to(dev), eps)
+    torch.cuda.synchronize()
+    return out.cpu(), s.cpu()
+
+
+@pytest.mark.parametrize('shape', [(2, 4, 2, torch.float32), (3, 8, 4, torch.bfloat16), (1, 16, 16, torch.float32),
+                                   (64, 32, 16, torch.bfloat16)])
+def test_fused_norm_matches_oracle(capi, dev, shape):
+    B, Hv, Hqk, dt = shape
+    gen = torch.Generator().manual_seed(400 + B)
+    ins = gdn.gdn_make_raw_inputs(B, Hv, Hqk, qkv_dtype=dt, generator=gen)
+    z = (torch.randn(B, Hv, 128, generator=gen) * 2).to(dt)
+    norm_w = (1.0 + 0.1 * torch.randn(128, generator=gen)).to(dt)
+    want, want_s = gdn.gdn_decode_fused_norm_step(*ins[:7], ins[7].clone(), z, norm_w)
+    out, s = run_fused_norm(capi, dev, ins, z, norm_w)
+    assert gdn.gdn_close(s, want_s)
+    assert out.dtype == dt
+    if dt == torch.float32:
+        assert gdn.gdn_close(out, want)
+    else:
+        # bf16 output: the oracle's value or its bf16 neighbour where the fp32 results straddle a rounding boundary
+        a_, b_ = out.float(), want.float()
+        assert ((a_ - b_).abs() <= torch.maximum(a_.abs(), b_.abs()) * 2.0 ** -7 + 1e-3 * b_.abs().max()).all()
+        assert (out == want).float().mean() >= 0.97
+    # the state is the plain fused step's, bit for bit, when that runs with the same tiling (config 9: one
+    # workgroup of 1024 lanes per head); the normalisation only touches the output
+    _, s_plain = run_fused(capi, dev, ins, 9)
+    assert torch.equal(s, s_plain)
+
+
+def test_fused_norm_equals_norm_of_the_fused_read_out(capi, dev):
+    gen = torch.Generator().manual_seed(45)
+    ins = gdn.gdn_make_raw_inputs(4, 8, 4, generator=gen)
+    z = torch.randn(4, 8, 128, generator=gen)
+    norm_w = 1.0 + 0.1 * torch.randn(128, generator=gen)
+    o, _ = run_fused(capi, dev, ins)
+    out, _ = run_fused_norm(capi, dev, ins, z, norm_w)
+    torch.testing.assert_close(out, gdn.gated_rmsnorm(o, z, norm_w), rtol=2e-5, atol=1e-6)
+
+
+def test_fused_norm_golden_fixture(capi, dev):
+    # the recurrence from the fused golden fixture, then the third-party norm module's own fixture shapes the norm
+    zf = np.load(FUSED_GOLDEN)
+    ins = [torch.from_numpy(zf[n]) for n in ('q', 'k', 'v', 'a', 'b', 'a_log', 'dt_bias', 'state')]
+    g = np.load(FUSED_GOLDEN.with_name('gated_rmsnorm_golden.npz'))
+    B, Hv = ins[2].shape[:2]
+    gen = torch.Generator().manual_seed(46)
+    z = torch.randn(B, Hv, 128, generator=gen)
+    norm_w = torch.from_numpy(g['weight'])
+    out, s = run_fused_norm(capi, dev, ins, z, norm_w)
+    want = gdn.gated_rmsnorm(torch.from_numpy(zf['o']), z, norm_w)
+    assert gdn.gdn_close(out, want) and gdn.gdn_close(s, torch.from_numpy(zf['new_state']))

@@ -241,3 +241,28 @@ def test_conv_update_rounds_once_for_bf16():
     out = gdn.causal_conv1d_update(x, state, weight, bias)
     assert out.dtype == torch.bfloat16 and state.dtype == torch.bfloat16
     assert torch.equal(out, exact.bfloat16())
+
+
+# ---- gated RMS normalisation of the read-out -----------------------------------------------------
+
+def test_gated_rmsnorm_closed_form_and_invariants():
+    gen = torch.Generator().manual_seed(12)
+    o = torch.randn(5, 7, 128, generator=gen) * 3
+    z = torch.randn(5, 7, 128, generator=gen)
+    w = 1.0 + 0.2 * torch.randn(128, generator=gen)
+    y = gdn.gated_rmsnorm(o, z, w, 1e-6)
+    od, zd = o.double(), z.double()
+    want = w.double() * od / torch.sqrt(od.pow(2).mean(-1, keepdim=True) + 1e-6) * zd / (1 + torch.exp(-zd))
+    torch.testing.assert_close(y.double(), want, rtol=1e-5, atol=1e-6)
+    # the normalised vector has unit rms; a zero gate gives zero; scale invariance in o (eps aside)
+    n = gdn.gated_rmsnorm(o, torch.full_like(z, 50.0), torch.ones(128), 0.0) / 50.0
+    torch.testing.assert_close(n.pow(2).mean(-1), torch.ones(5, 7), rtol=1e-5, atol=0)
+    assert (gdn.gated_rmsnorm(o, torch.zeros_like(z), w) == 0).all()
+    torch.testing.assert_close(gdn.gated_rmsnorm(4 * o, z, w, 0.0), gdn.gated_rmsnorm(o, z, w, 0.0), rtol=1e-5, atol=1e-6)
+    assert gdn.gated_rmsnorm(o, z.bfloat16(), w).dtype == torch.bfloat16
+
+
+def test_gated_rmsnorm_matches_third_party_golden():
+    g = np.load(GOLDEN_DIR / 'gated_rmsnorm_golden.npz')
+    y = gdn.gated_rmsnorm(torch.from_numpy(g['o']), torch.from_numpy(g['z']), torch.from_numpy(g['weight']), 1e-6)
+    np.testing.assert_allclose(y.numpy(), g['y'], rtol=1e-5, atol=1e-6)
