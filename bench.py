@@ -268,6 +268,37 @@ def bench_router(torch, capi, dev, steps, warmup, cpu_baseline, prefill):
     return res
 
 
+def bench_index_scores(torch, capi, dev, steps, warmup, cpu_baseline):
+    """The indexer scores in front of the selection: 64 requests, 64 index heads of 128, 32768 cached index keys
+    (bf16) per request."""
+    from oracle import mla
+    B, Hi, N = 64, 64, 32768
+    gen = torch.Generator(device=dev).manual_seed(20262)
+    q = torch.randn(B, Hi, 128, device=dev, generator=gen).bfloat16()
+    k = torch.randn(B, N, 128, device=dev, generator=gen).bfloat16()     # 537 MB: twice the last-level cache
+    w = torch.randn(B, Hi, device=dev, generator=gen) / 8
+    scores = torch.empty(B, N, device=dev)
+    sec = timed_launches(torch, lambda i: capi.mla_index_scores_launch(scores, q, k, w), steps, warmup)
+    work = B * N * 128 * 2 + B * N * 4 + B * Hi * 128 * 2 + B * Hi * 4
+    flops = 2 * B * Hi * N * 128
+    res = dict(
+        workload="indexer scores in front of configs[3]: B=64, 64 index heads x 128, 32768 bf16 index keys per "
+                 "request, seed 20262",
+        value=work / sec / 1e9, unit="GB/s", ms_per_step=sec * 1e3, dtype="bf16", kernel="mla_index_scores_kernel",
+        roofline=dict(bound="hbm", achieved=work / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
+                      frac=work / sec / 1e9 / HBM_PEAK_GBS, traffic=None),
+        algorithmic_bytes=work, tflops=flops / sec / 1e12)
+    if cpu_baseline:
+        cores = len(os.sched_getaffinity(0))
+        torch.set_num_threads(cores)
+        nb = 4
+        hq, hk, hw = q[:nb].cpu(), k[:nb].cpu(), w[:nb].cpu()
+        csec = cpu_time(lambda: mla.index_scores(hq, hk, hw))
+        res['cpu_baseline'] = dict(value=work / B * nb / csec / 1e9, unit="GB/s", cores=cores, kind="port",
+                                   sample="requests 0..3 (1/16 of the batch), eager PyTorch oracle")
+    return res
+
+
 def bench_topk_select(torch, capi, dev, steps, warmup, cpu_baseline):
     """The selection in front of configs[3]: 2048 of 32768 index scores per request, 64 requests."""
     from oracle import mla
@@ -462,7 +493,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=20)
     ap.add_argument('--warmup', type=int, default=5)
-    ap.add_argument('--workloads', default='gdn,gdn_fused,gdn_fused_norm,conv1d,moe_decode,router_decode,topk_select,mla,mla_paged,moe_prefill,router_prefill')
+    ap.add_argument('--workloads', default='gdn,gdn_fused,gdn_fused_norm,conv1d,moe_decode,router_decode,index_scores,topk_select,mla,mla_paged,moe_prefill,router_prefill')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run 3 plain device copies of 536 870 912 bytes (a kernel of known traffic, '
@@ -501,6 +532,8 @@ def main():
             results[name] = bench_conv1d(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name in ('router_decode', 'router_prefill'):
             results[name] = bench_router(torch, capi, dev, args.steps, args.warmup, cpu, name == 'router_prefill')
+        elif name == 'index_scores':
+            results[name] = bench_index_scores(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'topk_select':
             results[name] = bench_topk_select(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'mla':

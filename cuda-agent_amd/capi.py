@@ -33,6 +33,7 @@ SIGNATURES = {
                                                 _P]),
     'sparse_mla_decode_num_splits': (c_int, [c_int, c_int, c_int, c_int]),
     'sparse_mla_decode_workspace_bytes': (c_size_t, [c_int, c_int, c_int, c_int]),
+    'mla_index_scores_launcher': (None, [_P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_float, c_int, _P]),
     'topk_select_launcher': (None, [_P, _P, _P, c_int, c_int, c_int, c_int, _P]),
     'moe_route_launcher': (None, [_P, _P, _P, c_int, c_int, c_int, c_int, _P]),
     'moe_router_logits_num_splits': (c_int, [c_int, c_int, c_int]),
@@ -283,6 +284,27 @@ def sparse_mla_decode_paged_launch(out, q, kv_pool, block_table, idx, workspace,
         0 if out.dtype == torch.bfloat16 else 1, config, _stream(stream))
     check_status('sparse_mla_decode_paged_launcher')
     return out
+
+
+def mla_index_scores_launch(scores, q, k_cache, w, lengths=None, scale=128 ** -0.5, stream=None):
+    """scores [B, N] fp32 <- sum_h w[b,h] * relu(scale * q[b,h] . k_cache[b,t]); -inf at t >= lengths[b].
+    q [B, Hi, 128] bf16, k_cache [B, N, 128] bf16, w [B, Hi] fp32."""
+    import torch
+    _device_contiguous(scores=scores, q=q, k_cache=k_cache, w=w)
+    B, Hi, D = q.shape
+    N = k_cache.shape[1]
+    _require(q.dtype == k_cache.dtype == torch.bfloat16 and w.dtype == scores.dtype == torch.float32,
+             'mla_index_scores: q, k_cache bf16; w, scores fp32')
+    _require(tuple(k_cache.shape) == (B, N, D) and tuple(w.shape) == (B, Hi) and tuple(scores.shape) == (B, N),
+             'mla_index_scores: shapes')
+    if lengths is not None:
+        _device_contiguous(lengths=lengths)
+        _require(lengths.dtype == torch.int32 and tuple(lengths.shape) == (B,), 'mla_index_scores: lengths int32 [B]')
+    library().mla_index_scores_launcher(_ptr(scores), _ptr(q), _ptr(k_cache), _ptr(w),
+                                        _ptr(lengths) if lengths is not None else c_void_p(None), B, Hi, N, D,
+                                        float(scale), 0, _stream(stream))
+    check_status('mla_index_scores_launcher')
+    return scores
 
 
 def topk_select_launch(idx_out, scores, lengths=None, stream=None):

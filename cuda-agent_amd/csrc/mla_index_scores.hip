@@ -1,0 +1,156 @@
+// Index scores of the sparse-attention indexer, decode step: the scores whose top-k are the rows
+// sparse-MLA decode gathers. Per request b and cached position t:
+//
+//   score[b, t] = sum_h w[b, h] * max(0, scale * q[b, h, :] . k[b, t, :])       h over the index heads
+//
+// q [batch, n_heads, 128] and the index-key cache k [batch, n_rows, 128] are bf16, w [batch, n_heads]
+// fp32 (the per-head weights, with whatever normalisation the layer applies already in them);
+// positions at or beyond lengths[b] get -inf, so that a top-k over the row never selects them.
+//
+// The cache is read once (256 bytes per position) against 2 * n_heads * 128 flops per position: with
+// 64 heads the step is bound by HBM, so the kernel is a stream. A wavefront owns tiles of 32
+// positions: S = Q K^T on v_mfma_f32_32x32x16_bf16 with Q (heads x 128) resident in registers as the
+// A operand and the 32 cache rows as the B operand. In the 32x32 shapes any assignment of k to (lane
+// half, step) is valid as long as both operands use it, so lane (row, half) takes the contiguous 64
+// values [64*half, +64) of its row. The rows are fetched with whole lines per load instruction and
+// reach that layout through a small LDS buffer private to the wavefront (see the kernel); the next
+// tile's loads are in flight while the current tile is multiplied. In the result a lane holds 16
+// heads of one position per head tile: ReLU, weight and the sum over heads are in-lane, plus one
+// exchange between the two lane halves.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "launch_status.hpp"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int INDEX_DIM = 128;
+constexpr int K_STEPS = INDEX_DIM / 16;   // MFMAs per head tile and position tile
+constexpr int TILE_POS = 32;
+constexpr int TILES_PER_WAVE = 4;
+constexpr int WG_POS = 4 * TILES_PER_WAVE * TILE_POS;  // positions per workgroup of 4 wavefronts
+
+// grid: x = blocks of WG_POS positions, y = request. HT = n_heads / 32.
+template <int HT>
+__global__ __launch_bounds__(256) void mla_index_scores_kernel(
+    const __bf16* __restrict__ q, const __bf16* __restrict__ k_cache, const float* __restrict__ w,
+    const int* __restrict__ lengths, float* __restrict__ scores, int n_rows, float scale) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int row = lane & 31;
+    const int half = lane >> 5;
+    const int b = blockIdx.y;
+    const int n_heads = 32 * HT;
+    int valid = lengths != nullptr ? lengths[b] : n_rows;
+    valid = valid < 0 ? 0 : (valid > n_rows ? n_rows : valid);
+    const int first_tile = (blockIdx.x * 4 * TILES_PER_WAVE + wave * TILES_PER_WAVE) * TILE_POS;
+    if (first_tile >= n_rows) return;  // (no barrier in this kernel)
+
+    // Cache rows come in with whole lines per instruction (lane l of load j fetches 16-byte chunk
+    // l % 16 of row 4*j + l / 16 of the tile) and are turned into the operand layout (lane = row)
+    // through an 8 KB LDS buffer private to the wavefront: chunk c of row r sits at chunk slot
+    // c ^ (r % 16), which makes the 16 lanes that a write or a read instruction serves per cycle hit
+    // 16 different chunk slots. (Loading the operand layout directly asks the memory pipeline for 64
+    // different lines per instruction and ran at 2.2 TB/s.)
+    __shared__ u32x4 s_tile[4][TILE_POS * 16];
+    u32x4* tile = s_tile[wave];
+    const u32x4* kb = reinterpret_cast<const u32x4*>(k_cache + (size_t)b * n_rows * INDEX_DIM);
+    u32x4 raw[8];
+    auto load_tile = [&](int t0) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            int t = t0 + 4 * j + (lane >> 4);
+            t = t < n_rows ? t : n_rows - 1;  // rows past the end repeat the last one; not stored
+            raw[j] = __builtin_nontemporal_load(kb + (size_t)t * 16 + (lane & 15));
+        }
+    };
+    auto stage_tile = [&]() {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int r = 4 * j + (lane >> 4);
+            tile[r * 16 + ((lane & 15) ^ (r & 15))] = raw[j];
+        }
+    };
+    bf16x8 kf[K_STEPS];
+    auto read_operand = [&]() {
+#pragma unroll
+        for (int s = 0; s < K_STEPS; ++s)
+            kf[s] = __builtin_bit_cast(bf16x8, tile[row * 16 + ((8 * half + s) ^ (row & 15))]);
+    };
+    load_tile(first_tile);
+
+    // Q operand: head 32*ht + row, values [64*half + 8*s, +8) of step s; and this lane's weights:
+    // result register i of head tile ht is head 32*ht + 8*(i/4) + 4*half + i%4
+    bf16x8 qf[HT][K_STEPS];
+    floatx4 wf[HT][4];
+#pragma unroll
+    for (int ht = 0; ht < HT; ++ht) {
+        const bf16x8* src = reinterpret_cast<const bf16x8*>(
+            q + ((size_t)b * n_heads + 32 * ht + row) * INDEX_DIM + 64 * half);
+#pragma unroll
+        for (int s = 0; s < K_STEPS; ++s) qf[ht][s] = src[s];
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+            wf[ht][g] = *reinterpret_cast<const floatx4*>(w + (size_t)b * n_heads + 32 * ht + 8 * g + 4 * half);
+    }
+
+#pragma unroll
+    for (int i = 0; i < TILES_PER_WAVE; ++i) {
+        const int t0 = first_tile + i * TILE_POS;
+        if (t0 >= n_rows) break;
+        stage_tile();  // (LDS operations of a wavefront execute in order: no barrier, the buffer is private)
+        if (i + 1 < TILES_PER_WAVE && t0 + TILE_POS < n_rows) load_tile(t0 + TILE_POS);
+        read_operand();
+        float total = 0.f;
+#pragma unroll
+        for (int ht = 0; ht < HT; ++ht) {
+            floatx16 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < K_STEPS; ++s)
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qf[ht][s], kf[s], acc, 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < 16; ++j) total = fmaf(wf[ht][j / 4][j % 4], fmaxf(scale * acc[j], 0.f), total);
+        }
+        total += __shfl_xor(total, 32);
+        const int t = t0 + row;
+        if (half == 0 && t < n_rows) scores[(size_t)b * n_rows + t] = t < valid ? total : -INFINITY;
+    }
+}
+
+}  // namespace
+
+// scores [batch, n_rows] fp32, written: sum over heads of w * relu(scale * q . k) for positions below
+//        lengths[b] (all, if lengths is null), -inf beyond
+// q [batch, n_heads, 128] bf16; k_cache [batch, n_rows, 128] bf16; w [batch, n_heads] fp32;
+// lengths [batch] int32 or null. n_heads 32 or 64; q, k_cache and w 16-byte aligned.
+// config is accepted for the launcher pattern and has one value.
+extern "C" void mla_index_scores_launcher(float* scores, const void* q, const void* k_cache,
+                                          const float* w, const int* lengths, int batch,
+                                          int n_heads, int n_rows, int head_dim, float scale,
+                                          int config, hipStream_t stream) {
+    (void)config;
+    if (batch <= 0 || n_rows <= 0) return;
+    if ((n_heads != 32 && n_heads != 64) || head_dim != INDEX_DIM || batch > 65535) {
+        caa::set_status(CAA_UNSUPPORTED_SHAPE);
+        return;
+    }
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k_cache) |
+                           reinterpret_cast<uintptr_t>(w);
+    if (!scores || !q || !k_cache || !w || (bits & 15u) != 0) {
+        caa::set_status(CAA_BAD_ARGUMENT);
+        return;
+    }
+    const dim3 grid((n_rows + WG_POS - 1) / WG_POS, batch);
+    const __bf16* qb = static_cast<const __bf16*>(q);
+    const __bf16* kb = static_cast<const __bf16*>(k_cache);
+    if (n_heads == 32) {
+        mla_index_scores_kernel<1><<<grid, 256, 0, stream>>>(qb, kb, w, lengths, scores, n_rows, scale);
+    } else {
+        mla_index_scores_kernel<2><<<grid, 256, 0, stream>>>(qb, kb, w, lengths, scores, n_rows, scale);
+    }
+}

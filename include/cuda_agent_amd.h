@@ -166,6 +166,17 @@ int sparse_mla_decode_num_splits(int batch, int n_heads, int topk, int config);
 /* Bytes of workspace sparse_mla_decode_launcher needs for these sizes and this config. */
 size_t sparse_mla_decode_workspace_bytes(int batch, int n_heads, int topk, int config);
 
+/* Index scores of the sparse-attention indexer, decode step (caller-side neighbour of the top-k
+ * selection below; same launcher pattern agent_workdir/kernels/axpby.cu:12-20):
+ *   scores[b, t] = sum_h w[b, h] * max(0, scale * q[b, h, :] . k_cache[b, t, :])  for t < lengths[b]
+ *                  (all n_rows if lengths is NULL), -inf beyond
+ *   scores [batch, n_rows] fp32; q [batch, n_heads, 128] bf16; k_cache [batch, n_rows, 128] bf16;
+ *   w [batch, n_heads] fp32 (per-head weights, any normalisation already applied).
+ * n_heads 32 or 64, head_dim 128; q, k_cache, w 16-byte aligned. config: one value (0). */
+void mla_index_scores_launcher(float* scores, const void* q, const void* k_cache, const float* w,
+                               const int* lengths, int batch, int n_heads, int n_rows, int head_dim,
+                               float scale, int config, hipStream_t stream);
+
 /* Top-k selection of index scores, the step that produces idx for the two launchers above
  * (caller-side neighbour; same launcher pattern agent_workdir/kernels/axpby.cu:12-20):
  *   idx_out [batch, k] int32: per request the indices of the k largest scores among the first

@@ -25,6 +25,12 @@ one pool shared by all requests. Pinned by scalar loops over divmod on small cas
 identity "scatter a contiguous cache's pages into a pool under a random page permutation ->
 the paged result equals the contiguous result exactly".
 
+``index_scores`` is the scoring in front of the selection (the indexer of DeepSeek sparse attention on one
+decode step: per-head ReLU of scaled q.k, weighted sum over the index heads). Pinned by scalar loops in
+float64, by its invariants (non-negative weights give non-negative scores, a head with weight 0 drops out,
+scores are linear in w) and by a golden fixture from the third-party ``transformers`` indexer module, whose
+returned top-k indices must equal the top-k of these scores (tests/golden/make_indexer_golden.py).
+
 ``topk_select`` is the selection that produces ``idx`` from index scores. Pinned by ``torch.topk`` as
 a set on tie-free rows, by scalar loops with an explicit (value, index) ordering on rows full of
 ties, signed zeros, infinities and NaNs, and by its invariants (ascending indices, every chosen
@@ -125,6 +131,17 @@ def mla_scatter_into_pool(kv, page_size, n_spare_pages=3, generator=None):
     pool = torch.randn(n_pages, page_size, d, generator=generator).to(kv.dtype)
     pool[order] = kv.reshape(B * per_req, page_size, d).cpu()
     return pool, order.reshape(B, per_req).int()
+
+
+def index_scores(q, k_cache, w, lengths=None, scale=128 ** -0.5):
+    """Indexer scores of a decode step: q [B,Hi,d], k_cache [B,N,d] (bf16, taken to fp32), w [B,Hi] fp32 ->
+    scores [B,N] fp32 = sum_h w[b,h] * relu(scale * q[b,h] . k_cache[b,t]); -inf at positions >= lengths[b]."""
+    s = torch.einsum('bhd,bnd->bhn', q.float(), k_cache.float()) * scale
+    out = torch.einsum('bh,bhn->bn', w.float(), torch.relu(s))
+    if lengths is not None:
+        pos = torch.arange(k_cache.shape[1], device=out.device)[None, :]
+        out = out.masked_fill(pos >= lengths.to(out.device)[:, None].long(), float('-inf'))
+    return out
 
 
 def topk_select(scores, k, lengths=None):

@@ -182,3 +182,39 @@ def test_topk_select_ties_specials_and_lengths():
             unchosen = torch.ones(50, dtype=torch.bool)
             unchosen[row.long()] = False
             assert scores[b, row.long()].min() >= scores[b, unchosen].max()
+
+
+# ---- indexer scores ------------------------------------------------------------------------------
+
+def test_index_scores_match_float64_loops_and_invariants():
+    gen = torch.Generator().manual_seed(33)
+    B, Hi, N, d = 2, 4, 9, 16
+    q = torch.randn(B, Hi, d, generator=gen).bfloat16()
+    k = torch.randn(B, N, d, generator=gen).bfloat16()
+    w = torch.randn(B, Hi, generator=gen)
+    lengths = torch.tensor([9, 5], dtype=torch.int32)
+    got = mla.index_scores(q, k, w, lengths, scale=0.25)
+    for b in range(B):
+        for t in range(N):
+            if t >= int(lengths[b]):
+                assert got[b, t] == float('-inf')
+                continue
+            want = sum(float(w[b, h]) * max(0.0, 0.25 * sum(float(q[b, h, j]) * float(k[b, t, j]) for j in range(d)))
+                       for h in range(Hi))
+            assert abs(float(got[b, t]) - want) <= 1e-5 * (1 + abs(want))
+    assert (mla.index_scores(q, k, w.abs()) >= 0).all()
+    w0 = w.clone()
+    w0[:, 1] = 0
+    q_other = q.clone()
+    q_other[:, 1] = 7.0
+    assert torch.equal(mla.index_scores(q, k, w0), mla.index_scores(q_other, k, w0))       # a head of weight 0 drops out
+    torch.testing.assert_close(mla.index_scores(q, k, 3 * w), 3 * mla.index_scores(q, k, w), rtol=1e-6, atol=1e-6)
+
+
+def test_index_scores_select_what_the_third_party_indexer_selects():
+    from pathlib import Path
+    z = np.load(Path(__file__).parent / 'golden' / 'indexer_golden.npz')
+    q, k, w = (torch.from_numpy(z[n]) for n in ('q', 'k', 'w'))
+    scores = mla.index_scores(q, k, w, scale=float(z['scale'][0]))
+    idx = mla.topk_select(scores, z['topk'].shape[1])
+    np.testing.assert_array_equal(idx.numpy(), z['topk'])
