@@ -37,7 +37,7 @@ METRIC = "GB/s & % HBM peak (GDN/MoE/MLA decode); fp8 TFLOP/s % MFMA peak (MoE p
 # by the same counters read on a plain 512 MiB copy kernel (FETCH_SIZE x 1.99981, WRITE_SIZE x 1,
 # both in KiB); the counter summary is profiles/all_workloads_hbm_traffic_pmc.md.
 # None = not measured.
-MEASURED_TRAFFIC = {'gdn': 1085972770, 'moe_decode': 6664643628, 'mla': 256686692, 'moe_prefill': 11230161000}
+MEASURED_TRAFFIC = {'gdn': 1085972770, 'moe_decode': 6664643628, 'mla': 223278459, 'index_scores': 553871480, 'moe_prefill': 11230161000}
 
 
 SETTLE_SECONDS = 0.05
@@ -286,7 +286,7 @@ def bench_index_scores(torch, capi, dev, steps, warmup, cpu_baseline):
                  "request, seed 20262",
         value=work / sec / 1e9, unit="GB/s", ms_per_step=sec * 1e3, dtype="bf16", kernel="mla_index_scores_kernel",
         roofline=dict(bound="hbm", achieved=work / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
-                      frac=work / sec / 1e9 / HBM_PEAK_GBS, traffic=None),
+                      frac=work / sec / 1e9 / HBM_PEAK_GBS, traffic=MEASURED_TRAFFIC['index_scores']),
         algorithmic_bytes=work, tflops=flops / sec / 1e12)
     if cpu_baseline:
         cores = len(os.sched_getaffinity(0))
