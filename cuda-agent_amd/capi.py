@@ -34,6 +34,8 @@ SIGNATURES = {
     'sparse_mla_decode_num_splits': (c_int, [c_int, c_int, c_int, c_int]),
     'sparse_mla_decode_workspace_bytes': (c_size_t, [c_int, c_int, c_int, c_int]),
     'mla_index_scores_launcher': (None, [_P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_float, c_int, _P]),
+    'mla_index_scores_paged_launcher': (None, [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int,
+                                               c_float, c_int, _P]),
     'topk_select_launcher': (None, [_P, _P, _P, c_int, c_int, c_int, c_int, _P]),
     'moe_route_launcher': (None, [_P, _P, _P, c_int, c_int, c_int, c_int, _P]),
     'moe_router_logits_num_splits': (c_int, [c_int, c_int, c_int]),
@@ -304,6 +306,30 @@ def mla_index_scores_launch(scores, q, k_cache, w, lengths=None, scale=128 ** -0
                                         _ptr(lengths) if lengths is not None else c_void_p(None), B, Hi, N, D,
                                         float(scale), 0, _stream(stream))
     check_status('mla_index_scores_launcher')
+    return scores
+
+
+def mla_index_scores_paged_launch(scores, q, k_pool, block_table, w, lengths=None, scale=128 ** -0.5, stream=None):
+    """As ``mla_index_scores_launch`` over a paged key cache: k_pool [n_pages, page, 128] bf16, block_table
+    [B, max_pages] int32; scores [B, max_pages * page] over logical positions."""
+    import torch
+    _device_contiguous(scores=scores, q=q, k_pool=k_pool, block_table=block_table, w=w)
+    B, Hi, D = q.shape
+    n_pages, page = k_pool.shape[0], k_pool.shape[1]
+    max_pages = block_table.shape[1]
+    _require(q.dtype == k_pool.dtype == torch.bfloat16 and w.dtype == scores.dtype == torch.float32,
+             'mla_index_scores: q, k_pool bf16; w, scores fp32')
+    _require(block_table.dtype == torch.int32 and block_table.shape[0] == B, 'mla_index_scores: block_table int32 [B, P]')
+    _require(tuple(k_pool.shape) == (n_pages, page, D) and tuple(w.shape) == (B, Hi)
+             and tuple(scores.shape) == (B, max_pages * page), 'mla_index_scores: shapes')
+    if lengths is not None:
+        _device_contiguous(lengths=lengths)
+        _require(lengths.dtype == torch.int32 and tuple(lengths.shape) == (B,), 'mla_index_scores: lengths int32 [B]')
+    library().mla_index_scores_paged_launcher(
+        _ptr(scores), _ptr(q), _ptr(k_pool), _ptr(block_table), _ptr(w),
+        _ptr(lengths) if lengths is not None else c_void_p(None), B, Hi, n_pages, page, max_pages, D, float(scale),
+        0, _stream(stream))
+    check_status('mla_index_scores_paged_launcher')
     return scores
 
 

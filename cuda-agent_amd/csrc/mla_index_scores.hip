@@ -39,7 +39,11 @@ constexpr int WG_POS = 4 * TILES_PER_WAVE * TILE_POS;  // positions per workgrou
 template <int HT>
 __global__ __launch_bounds__(256) void mla_index_scores_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ k_cache, const float* __restrict__ w,
-    const int* __restrict__ lengths, float* __restrict__ scores, int n_rows, float scale) {
+    const int* __restrict__ lengths, float* __restrict__ scores, int n_rows, float scale,
+    const int* __restrict__ block_table, int table_stride, int page_shift, int pool_rows) {
+    // block_table == null: position t of request b is row b * n_rows + t of k_cache. Otherwise k_cache is
+    // a pool of pages shared by all requests and position t is row t % page of page
+    // block_table[b * table_stride + t / page]; positions of unmapped pages score -inf.
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int row = lane & 31;
@@ -59,14 +63,21 @@ __global__ __launch_bounds__(256) void mla_index_scores_kernel(
     // different lines per instruction and ran at 2.2 TB/s.)
     __shared__ u32x4 s_tile[4][TILE_POS * 16];
     u32x4* tile = s_tile[wave];
-    const u32x4* kb = reinterpret_cast<const u32x4*>(k_cache + (size_t)b * n_rows * INDEX_DIM);
+    const u32x4* kb = reinterpret_cast<const u32x4*>(k_cache) +
+                      (block_table == nullptr ? (size_t)b * n_rows * 16 : 0);
     u32x4 raw[8];
     auto load_tile = [&](int t0) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             int t = t0 + 4 * j + (lane >> 4);
             t = t < n_rows ? t : n_rows - 1;  // rows past the end repeat the last one; not stored
-            raw[j] = __builtin_nontemporal_load(kb + (size_t)t * 16 + (lane & 15));
+            size_t r = (size_t)t;
+            if (block_table != nullptr) {
+                const int page = block_table[(size_t)b * table_stride + (t >> page_shift)];
+                const long long pr = ((long long)page << page_shift) + (t & ((1 << page_shift) - 1));
+                r = (page >= 0 && pr < pool_rows) ? (size_t)pr : 0;  // unmapped: any row, masked below
+            }
+            raw[j] = __builtin_nontemporal_load(kb + r * 16 + (lane & 15));
         }
     };
     auto stage_tile = [&]() {
@@ -118,22 +129,25 @@ __global__ __launch_bounds__(256) void mla_index_scores_kernel(
         }
         total += __shfl_xor(total, 32);
         const int t = t0 + row;
-        if (half == 0 && t < n_rows) scores[(size_t)b * n_rows + t] = t < valid ? total : -INFINITY;
+        if (half == 0 && t < n_rows) {
+            bool live = t < valid;
+            if (live && block_table != nullptr) {
+                const int page = block_table[(size_t)b * table_stride + (t >> page_shift)];
+                live = page >= 0 && (((long long)page << page_shift) + (t & ((1 << page_shift) - 1))) < pool_rows;
+            }
+            scores[(size_t)b * n_rows + t] = live ? total : -INFINITY;
+        }
     }
 }
 
 }  // namespace
 
-// scores [batch, n_rows] fp32, written: sum over heads of w * relu(scale * q . k) for positions below
-//        lengths[b] (all, if lengths is null), -inf beyond
-// q [batch, n_heads, 128] bf16; k_cache [batch, n_rows, 128] bf16; w [batch, n_heads] fp32;
-// lengths [batch] int32 or null. n_heads 32 or 64; q, k_cache and w 16-byte aligned.
-// config is accepted for the launcher pattern and has one value.
-extern "C" void mla_index_scores_launcher(float* scores, const void* q, const void* k_cache,
-                                          const float* w, const int* lengths, int batch,
-                                          int n_heads, int n_rows, int head_dim, float scale,
-                                          int config, hipStream_t stream) {
-    (void)config;
+namespace {
+
+void launch_index_scores(float* scores, const void* q, const void* k_cache, const float* w,
+                         const int* lengths, int batch, int n_heads, int n_rows, int head_dim,
+                         float scale, const int* block_table, int table_stride, int page_shift,
+                         int pool_rows, hipStream_t stream) {
     if (batch <= 0 || n_rows <= 0) return;
     if ((n_heads != 32 && n_heads != 64) || head_dim != INDEX_DIM || batch > 65535) {
         caa::set_status(CAA_UNSUPPORTED_SHAPE);
@@ -149,8 +163,56 @@ extern "C" void mla_index_scores_launcher(float* scores, const void* q, const vo
     const __bf16* qb = static_cast<const __bf16*>(q);
     const __bf16* kb = static_cast<const __bf16*>(k_cache);
     if (n_heads == 32) {
-        mla_index_scores_kernel<1><<<grid, 256, 0, stream>>>(qb, kb, w, lengths, scores, n_rows, scale);
+        mla_index_scores_kernel<1><<<grid, 256, 0, stream>>>(qb, kb, w, lengths, scores, n_rows, scale,
+                                                             block_table, table_stride, page_shift, pool_rows);
     } else {
-        mla_index_scores_kernel<2><<<grid, 256, 0, stream>>>(qb, kb, w, lengths, scores, n_rows, scale);
+        mla_index_scores_kernel<2><<<grid, 256, 0, stream>>>(qb, kb, w, lengths, scores, n_rows, scale,
+                                                             block_table, table_stride, page_shift, pool_rows);
     }
+}
+
+}  // namespace
+
+// scores [batch, n_rows] fp32, written: sum over heads of w * relu(scale * q . k) for positions below
+//        lengths[b] (all, if lengths is null), -inf beyond
+// q [batch, n_heads, 128] bf16; k_cache [batch, n_rows, 128] bf16; w [batch, n_heads] fp32;
+// lengths [batch] int32 or null. n_heads 32 or 64; q, k_cache and w 16-byte aligned.
+// config is accepted for the launcher pattern and has one value.
+extern "C" void mla_index_scores_launcher(float* scores, const void* q, const void* k_cache,
+                                          const float* w, const int* lengths, int batch,
+                                          int n_heads, int n_rows, int head_dim, float scale,
+                                          int config, hipStream_t stream) {
+    (void)config;
+    launch_index_scores(scores, q, k_cache, w, lengths, batch, n_heads, n_rows, head_dim, scale, nullptr,
+                        0, 0, 0, stream);
+}
+
+// The same scores over a paged index-key cache: k_pool [n_pages, page_size, 128] bf16 shared by all
+// requests, block_table [batch, max_pages_per_request] int32 (negative = not mapped). Position t of
+// request b is row t % page_size of page block_table[b][t / page_size]; scores has
+// max_pages_per_request * page_size columns, -inf at positions >= lengths[b] and at unmapped pages.
+// page_size a power of two, n_pages * page_size < 2^31.
+extern "C" void mla_index_scores_paged_launcher(float* scores, const void* q, const void* k_pool,
+                                                const int* block_table, const float* w,
+                                                const int* lengths, int batch, int n_heads,
+                                                int n_pages, int page_size, int max_pages_per_request,
+                                                int head_dim, float scale, int config,
+                                                hipStream_t stream) {
+    (void)config;
+    if (batch <= 0) return;
+    if (n_pages <= 0 || page_size <= 0 || (page_size & (page_size - 1)) != 0 || max_pages_per_request <= 0 ||
+        (long long)n_pages * page_size > 0x7fffffffll ||
+        (long long)max_pages_per_request * page_size > 0x7fffffffll) {
+        caa::set_status(CAA_UNSUPPORTED_SHAPE);
+        return;
+    }
+    if (!block_table) {
+        caa::set_status(CAA_BAD_ARGUMENT);
+        return;
+    }
+    int page_shift = 0;
+    while ((1 << page_shift) < page_size) ++page_shift;
+    launch_index_scores(scores, q, k_pool, w, lengths, batch, n_heads, max_pages_per_request * page_size,
+                        head_dim, scale, block_table, max_pages_per_request, page_shift,
+                        n_pages * page_size, stream);
 }

@@ -177,6 +177,18 @@ void mla_index_scores_launcher(float* scores, const void* q, const void* k_cache
                                const int* lengths, int batch, int n_heads, int n_rows, int head_dim,
                                float scale, int config, hipStream_t stream);
 
+/* The same scores over a paged index-key cache: k_pool [n_pages, page_size, 128] bf16 shared by
+ * all requests and block_table [batch, max_pages_per_request] int32 (negative = not mapped);
+ * position t of request b is row t % page_size of page block_table[b][t / page_size]. scores
+ * [batch, max_pages_per_request * page_size], -inf at positions >= lengths[b] and on unmapped pages:
+ * logical positions, as sparse_mla_decode_paged_launcher takes them with a block table. page_size a
+ * power of two; n_pages * page_size and max_pages_per_request * page_size below 2^31. */
+void mla_index_scores_paged_launcher(float* scores, const void* q, const void* k_pool,
+                                     const int* block_table, const float* w, const int* lengths,
+                                     int batch, int n_heads, int n_pages, int page_size,
+                                     int max_pages_per_request, int head_dim, float scale, int config,
+                                     hipStream_t stream);
+
 /* Top-k selection of index scores, the step that produces idx for the two launchers above
  * (caller-side neighbour; same launcher pattern agent_workdir/kernels/axpby.cu:12-20):
  *   idx_out [batch, k] int32: per request the indices of the k largest scores among the first

@@ -109,3 +109,33 @@ def test_rejects_unsupported_shapes(capi, dev):
     q, k, w = make(1, 48, 64, 1)
     with pytest.raises(capi.LaunchRejected):
         run_kernel(capi, dev, q, k, w)
+
+
+def test_paged_key_cache(capi, dev):
+    # the pages of a contiguous cache scattered into a pool: the same scores, bit for bit, on mapped pages;
+    # -inf on an unmapped page and beyond the lengths; then the whole paged chain scores -> selection -> attention
+    gen = torch.Generator().manual_seed(11)
+    B, H, Hi, N, page, topk = 3, 128, 64, 1024, 64, 200
+    q_idx, k_idx, w = make(B, Hi, N, 12)
+    q, kv, _ = mla.mla_make_inputs(B, H, N, topk, generator=gen)
+    k_pool, table = mla.mla_scatter_into_pool(k_idx, page, generator=gen)
+    kv_pool = torch.randn(k_pool.shape[0], page, 576, generator=gen).bfloat16()
+    kv_pool[table.reshape(-1).long()] = kv.reshape(-1, page, 576)            # the latent cache shares the block table
+    lengths = torch.tensor([N, 700, 333], dtype=torch.int32)
+    want = run_kernel(capi, dev, q_idx, k_idx, w, lengths)
+    table[1, 2] = -1
+    want[1, 128:192] = float('-inf')
+    scores = torch.full((B, N), float('nan'), device=dev)
+    capi.mla_index_scores_paged_launch(scores, q_idx.to(dev), k_pool.to(dev), table.to(dev), w.to(dev), lengths.to(dev))
+    torch.cuda.synchronize()
+    assert torch.equal(scores.cpu(), want)
+    idx = torch.empty(B, topk, dtype=torch.int32, device=dev)
+    out = torch.empty(B, H, 512, device=dev)
+    ws = torch.empty(capi.sparse_mla_workspace_bytes(B, H, topk), dtype=torch.uint8, device=dev)
+    capi.topk_select_launch(idx, scores, lengths.to(dev))
+    capi.sparse_mla_decode_paged_launch(out, q.to(dev), kv_pool.to(dev), table.to(dev), idx, ws)
+    torch.cuda.synchronize()
+    want_idx = mla.topk_select(want, topk, lengths)
+    assert torch.equal(idx.cpu(), want_idx)
+    ref = mla.sparse_mla_decode_paged(q, kv_pool, table, want_idx, out_dtype=torch.float32)
+    assert mla.rel_rms_error(out.cpu(), ref) <= 2e-2
