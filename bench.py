@@ -120,6 +120,33 @@ def bench_gdn(torch, capi, dev, steps, warmup, cpu_baseline):
     return res
 
 
+def bench_gdn_single(torch, capi, dev, steps, warmup, cpu_baseline):
+    """configs[0]: one request, 16 heads, fp32 q/k/v: 2 MB of state, a latency measurement (no target)."""
+    from oracle import gdn
+    B, Hv, Hqk = 1, 16, 16
+    gen = torch.Generator().manual_seed(20250)
+    host = gdn.gdn_make_inputs(B, Hv, Hqk, qkv_dtype=torch.float32, generator=gen)
+    q, k, v, g, beta, state0 = (t.to(dev) for t in host)
+    sets = [(torch.empty(B, Hv, 128, device=dev), state0.clone()) for _ in range(3)]
+    sec = timed_launches(torch, lambda i: capi.gdn_decode_launch(*sets[i % 3], q, k, v, g, beta), steps, warmup)
+    work = 2 * B * Hv * 128 * 128 * 4 + 3 * B * Hv * 128 * 4 + 2 * B * Hv * 4 + B * Hv * 128 * 4
+    res = dict(
+        workload="configs[0]: GDN single-request decode B=1, 16 heads, dk=dv=128, fp32, seed 20250 (1 MB of state "
+                 "read and written: launch latency, not bandwidth, sets the time)",
+        value=work / sec / 1e9, unit="GB/s", ms_per_step=sec * 1e3, dtype="f32", kernel="gdn_decode_kernel",
+        roofline=dict(bound="hbm", achieved=work / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
+                      frac=work / sec / 1e9 / HBM_PEAK_GBS, traffic=None),
+        algorithmic_bytes=work)
+    if cpu_baseline:
+        cores = len(os.sched_getaffinity(0))
+        torch.set_num_threads(cores)
+        csec = cpu_time(lambda: gdn.gdn_decode_step(*host), min_seconds=1.0, max_iters=200)
+        res['cpu_baseline'] = dict(value=work / csec / 1e9, unit="GB/s", cores=cores, kind="port",
+                                   sample="the full configs[0] step (eager PyTorch oracle, state in place), the case "
+                                          "the workload definition names as CPU-runnable")
+    return res
+
+
 def bench_gdn_fused_norm(torch, capi, dev, steps, warmup, cpu_baseline):
     """configs[1] sizes through the launcher that does the pre-step, the recurrence and the gated RMS
     normalisation of the read-out: the gate z is read (bf16) and the output is bf16 instead of fp32."""
@@ -493,7 +520,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=20)
     ap.add_argument('--warmup', type=int, default=5)
-    ap.add_argument('--workloads', default='gdn,gdn_fused,gdn_fused_norm,conv1d,moe_decode,router_decode,index_scores,topk_select,mla,mla_paged,moe_prefill,router_prefill')
+    ap.add_argument('--workloads', default='gdn,gdn_single,gdn_fused,gdn_fused_norm,conv1d,moe_decode,router_decode,index_scores,topk_select,mla,mla_paged,moe_prefill,router_prefill')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run 3 plain device copies of 536 870 912 bytes (a kernel of known traffic, '
@@ -526,6 +553,8 @@ def main():
             results[name] = bench_gdn(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'gdn_fused':
             results[name] = bench_gdn_fused(torch, capi, dev, args.steps, args.warmup, cpu)
+        elif name == 'gdn_single':
+            results[name] = bench_gdn_single(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'gdn_fused_norm':
             results[name] = bench_gdn_fused_norm(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'conv1d':
