@@ -295,6 +295,35 @@ def bench_router(torch, capi, dev, steps, warmup, cpu_baseline, prefill):
     return res
 
 
+def bench_rmsnorm_quant(torch, capi, dev, steps, warmup, cpu_baseline):
+    """The norm in front of configs[4] fused with the layer's quantiser: 8192 rows of 7168 bf16."""
+    from oracle import moe
+    T, H = 8192, 7168
+    gen = torch.Generator(device=dev).manual_seed(20263)
+    xs = [torch.randn(T, H, device=dev, generator=gen).bfloat16() for _ in range(3)]     # 3 x 117 MB
+    w = (1.0 + 0.1 * torch.randn(H, device=dev, generator=gen)).bfloat16()
+    q = torch.empty(T, H, dtype=torch.uint8, device=dev)
+    sc = torch.empty(T, H // 128, device=dev)
+    y = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    sec = timed_launches(torch, lambda i: capi.moe_rmsnorm_quant_launch(q, sc, y, xs[i % 3], w), steps, warmup)
+    work = T * H * (2 + 2 + 1) + T * (H // 128) * 4 + H * 2
+    res = dict(
+        workload="RMS norm + activation quantiser in front of configs[4]: 8192 x 7168 bf16 in; bf16 normalised rows, "
+                 "e4m3 codes and group scales out, seed 20263",
+        value=work / sec / 1e9, unit="GB/s", ms_per_step=sec * 1e3, dtype="f32", kernel="moe_rmsnorm_quant_kernel",
+        roofline=dict(bound="hbm", achieved=work / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
+                      frac=work / sec / 1e9 / HBM_PEAK_GBS, traffic=None),
+        algorithmic_bytes=work)
+    if cpu_baseline:
+        cores = len(os.sched_getaffinity(0))
+        torch.set_num_threads(cores)
+        hx, hw = xs[0][:1024].cpu(), w.cpu()
+        csec = cpu_time(lambda: moe.quantize_groups(moe.rmsnorm_bf16(hx, hw).float()))
+        res['cpu_baseline'] = dict(value=work / 8 / csec / 1e9, unit="GB/s", cores=cores, kind="port",
+                                   sample="rows 0..1023 (1/8), eager PyTorch oracle")
+    return res
+
+
 def bench_index_scores(torch, capi, dev, steps, warmup, cpu_baseline):
     """The indexer scores in front of the selection: 64 requests, 64 index heads of 128, 32768 cached index keys
     (bf16) per request."""
@@ -520,7 +549,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=20)
     ap.add_argument('--warmup', type=int, default=5)
-    ap.add_argument('--workloads', default='gdn,gdn_single,gdn_fused,gdn_fused_norm,conv1d,moe_decode,router_decode,index_scores,topk_select,mla,mla_paged,moe_prefill,router_prefill')
+    ap.add_argument('--workloads', default='gdn,gdn_single,gdn_fused,gdn_fused_norm,conv1d,moe_decode,router_decode,index_scores,topk_select,mla,mla_paged,moe_prefill,router_prefill,rmsnorm_quant')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run 3 plain device copies of 536 870 912 bytes (a kernel of known traffic, '
@@ -561,6 +590,8 @@ def main():
             results[name] = bench_conv1d(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name in ('router_decode', 'router_prefill'):
             results[name] = bench_router(torch, capi, dev, args.steps, args.warmup, cpu, name == 'router_prefill')
+        elif name == 'rmsnorm_quant':
+            results[name] = bench_rmsnorm_quant(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'index_scores':
             results[name] = bench_index_scores(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'topk_select':

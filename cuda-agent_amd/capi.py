@@ -46,6 +46,7 @@ SIGNATURES = {
     'moe_sort_launcher': (None, [_P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P]),
     'moe_route_sort_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P]),
     'moe_quant_bf16_launcher': (None, [_P, _P, _P, c_int, c_int, c_int, _P]),
+    'moe_rmsnorm_quant_launcher': (None, [_P, _P, _P, _P, _P, c_float, c_int, c_int, c_int, _P]),
     'moe_gate_up_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int,
                                     c_int, _P]),
     'moe_down_launcher': (None, [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P]),
@@ -471,6 +472,23 @@ def moe_quant_bf16_launch(q, scales, x, stream=None, config=0):
     library().moe_quant_bf16_launcher(_ptr(q), _ptr(scales), _ptr(x), R, C, config, _stream(stream))
     check_status('moe_quant_bf16_launcher')
     return q, scales
+
+
+def moe_rmsnorm_quant_launch(q, scales, y, x, weight, eps=1e-6, config=0, stream=None):
+    """y (bf16 or None) = RMS norm of x [R, C] bf16 with weight [C] bf16; q, scales = its activation quantisation."""
+    import torch
+    _device_contiguous(q=q, scales=scales, x=x, weight=weight)
+    R, C = x.shape
+    _require(x.dtype == weight.dtype == torch.bfloat16 and scales.dtype == torch.float32, 'moe_rmsnorm_quant: dtypes')
+    _require(q.element_size() == 1 and tuple(q.shape) == (R, C) and tuple(scales.shape) == (R, C // 128)
+             and tuple(weight.shape) == (C,), 'moe_rmsnorm_quant: shapes')
+    if y is not None:
+        _device_contiguous(y=y)
+        _require(y.dtype == torch.bfloat16 and tuple(y.shape) == (R, C), 'moe_rmsnorm_quant: y bf16 [R, C]')
+    library().moe_rmsnorm_quant_launcher(_ptr(q), _ptr(scales), _ptr(y) if y is not None else c_void_p(None),
+                                         _ptr(x), _ptr(weight), float(eps), R, C, config, _stream(stream))
+    check_status('moe_rmsnorm_quant_launcher')
+    return q, scales, y
 
 
 def moe_fp8_launch(out, x, logits, w13_q, w13_s, w2_q, w2_s, workspace, top_k=8, config=0, stream=None):

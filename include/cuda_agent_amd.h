@@ -262,6 +262,16 @@ void moe_route_sort_launcher(int* ids, float* weights, int* sorted_pairs, int* p
 void moe_quant_bf16_launcher(void* q, float* scales, const void* x, int rows, int cols, int config,
                              hipStream_t stream);
 
+/* The RMS norm in front of the layer fused with that quantiser (caller-side neighbour; same launcher
+ * pattern): y = weight * bf16(x * rsqrt(mean(x^2) + eps)) rounded to bf16 (the two roundings of a bf16
+ * norm layer), then q, scales = the quantisation above applied to y.
+ *   x [rows, cols] bf16, weight [cols] bf16, y [rows, cols] bf16 or NULL (the normalised row, e.g. for
+ *   the router projection), q [rows, cols] e4m3 codes, scales [rows, cols/128] fp32.
+ * cols a multiple of 128, at most 8192; x, weight, y 16-byte and q 8-byte aligned. config bit 32:
+ * power-of-two scales. */
+void moe_rmsnorm_quant_launcher(void* q, float* scales, void* y, const void* x, const void* weight,
+                                float eps, int rows, int cols, int config, hipStream_t stream);
+
 /* Grouped gate/up GEMM with SiLU(gate)*up and requantisation fused:
  * h_q [tokens*top_k, inter] e4m3, h_s [tokens*top_k, inter/128] fp32, rows in sorted order.
  * config: 0 sizes the pass from the average pairs per expert; 1, 2, 4 force 16, 32, 64 pairs

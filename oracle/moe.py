@@ -26,7 +26,10 @@ choice with a selection bias; no counterpart in the reference repository). Pinne
 on small sizes, by the reduction to ``route`` when there is one group and no bias, by its
 invariants (chosen experts lie in exactly topk_group groups, weights sum to the scaling factor),
 and by a golden fixture written from the third-party ``transformers`` router
-(tests/golden/make_router_golden.py). ``router_logits`` is the projection in front of it, pinned by a float64
+(tests/golden/make_router_golden.py). ``rmsnorm_bf16`` is the norm in front of the layer (its output is what the layer quantises and what the router
+projects); pinned by a float64 closed form within bf16 rounding and by a fixture from the third-party
+``DeepseekV3RMSNorm`` module in bf16 (``rmsnorm_golden.npz``, same generator script as the router's).
+``router_logits`` is the projection in front of it, pinned by a float64
 product and by the same fixture's logits.
 
 ``moe_forward_shared`` adds the shared expert of such a layer; it is built from ``moe_forward`` itself
@@ -143,6 +146,14 @@ def route(logits, top_k=8):
     order = torch.sort(logits, dim=-1, descending=True, stable=True).indices[:, :top_k]
     score = torch.sigmoid(logits.float()).gather(1, order)
     return order.int(), score / score.sum(dim=-1, keepdim=True)
+
+
+def rmsnorm_bf16(x, weight, eps=1e-6):
+    """The RMS norm of a bf16 layer as the third-party layers evaluate it: fp32 statistics, the normalised value
+    rounded to bf16, times the bf16 weight, rounded to bf16. x [R,C] bf16, weight [C] bf16 -> [R,C] bf16."""
+    xf = x.float()
+    n = (xf * (1.0 / torch.sqrt(xf.pow(2).mean(dim=-1, keepdim=True) + eps))).to(x.dtype)
+    return weight * n
 
 
 def router_logits(x, w):

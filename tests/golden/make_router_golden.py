@@ -40,6 +40,18 @@ def main():
     np.savez_compressed(out, **arrays)
     print('wrote', out, out.stat().st_size, 'bytes')
 
+    # the bf16 RMS norm in front of the layer
+    from transformers.models.deepseek_v3.modeling_deepseek_v3 import DeepseekV3RMSNorm
+    gen = torch.Generator().manual_seed(494949)
+    norm = DeepseekV3RMSNorm(256, eps=1e-6).bfloat16()
+    with torch.no_grad():
+        norm.weight.copy_((1.0 + 0.2 * torch.randn(256, generator=gen)).bfloat16())
+        x = (torch.randn(12, 256, generator=gen) * torch.exp(torch.randn(12, 1, generator=gen))).bfloat16()
+        y = norm(x)
+    out = Path(__file__).with_name('rmsnorm_golden.npz')
+    np.savez_compressed(out, x=x.float().numpy(), weight=norm.weight.detach().float().numpy(), y=y.float().numpy())
+    print('wrote', out, out.stat().st_size, 'bytes')
+
 
 if __name__ == '__main__':
     main()

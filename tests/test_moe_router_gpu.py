@@ -186,3 +186,56 @@ def test_router_logits_rejects_bad_arguments(capi, dev):
     with pytest.raises(capi.LaunchRejected):          # K is split for 4 tokens: scratch needed
         capi.moe_router_logits_launch(logits, torch.zeros(4, 7168, device=dev), w)
     torch.cuda.synchronize()
+
+
+# ---- RMS norm fused with the activation quantiser -------------------------------------------------
+
+@pytest.mark.parametrize('shape', [(64, 7168), (5, 128), (300, 2048), (1, 8192), (33, 384)])
+@pytest.mark.parametrize('config', [0, 32])
+def test_rmsnorm_quant(capi, dev, shape, config):
+    R, C = shape
+    gen = torch.Generator().manual_seed(R + C)
+    x = (torch.randn(R, C, generator=gen) * torch.exp(torch.randn(R, 1, generator=gen))).bfloat16()
+    w = (1.0 + 0.2 * torch.randn(C, generator=gen)).bfloat16()
+    q = torch.empty(R, C, dtype=torch.uint8, device=dev)
+    s = torch.empty(R, C // 128, device=dev)
+    y = torch.empty(R, C, dtype=torch.bfloat16, device=dev)
+    capi.moe_rmsnorm_quant_launch(q, s, y, x.to(dev), w.to(dev), 1e-6, config)
+    torch.cuda.synchronize()
+    # the normalised row: the oracle's bf16 value, or its neighbour where the fp32 sums of squares differ in the
+    # last place (different order of the additions) and the value sits on a bf16 rounding boundary
+    want_y = moe.rmsnorm_bf16(x, w)
+    assert (y.cpu() == want_y).float().mean().item() >= 0.995
+    assert ((y.cpu().float() - want_y.float()).abs() <= want_y.float().abs() * 2.0 ** -7).all()
+    # the quantisation of the kernel's own y: bit-exact
+    want_q, want_s = moe.quantize_groups(y.cpu().float(), pow2=config == 32)
+    assert torch.equal(s.cpu(), want_s)
+    assert torch.equal(q.cpu(), want_q.view(torch.uint8))
+    # y is optional
+    q2 = torch.empty_like(q)
+    s2 = torch.empty_like(s)
+    capi.moe_rmsnorm_quant_launch(q2, s2, None, x.to(dev), w.to(dev), 1e-6, config)
+    torch.cuda.synchronize()
+    assert torch.equal(q2, q) and torch.equal(s2, s)
+
+
+def test_rmsnorm_quant_golden_fixture(capi, dev):
+    z = np.load(Path(__file__).parent / 'golden' / 'rmsnorm_golden.npz')
+    x, w = torch.from_numpy(z['x']).bfloat16(), torch.from_numpy(z['weight']).bfloat16()
+    R, C = x.shape
+    q = torch.empty(R, C, dtype=torch.uint8, device=dev)
+    s = torch.empty(R, C // 128, device=dev)
+    y = torch.empty(R, C, dtype=torch.bfloat16, device=dev)
+    capi.moe_rmsnorm_quant_launch(q, s, y, x.to(dev), w.to(dev))
+    torch.cuda.synchronize()
+    want = torch.from_numpy(z['y'])
+    assert (y.cpu().float() == want).float().mean().item() >= 0.995
+    assert ((y.cpu().float() - want).abs() <= want.abs() * 2.0 ** -7).all()
+
+
+def test_rmsnorm_quant_rejects_bad_shapes(capi, dev):
+    x = torch.zeros(2, 8320, dtype=torch.bfloat16, device=dev)        # more than 8192 columns
+    with pytest.raises(capi.LaunchRejected):
+        capi.moe_rmsnorm_quant_launch(torch.empty(2, 8320, dtype=torch.uint8, device=dev),
+                                      torch.empty(2, 65, device=dev), None, x, torch.zeros(8320, dtype=torch.bfloat16, device=dev))
+    torch.cuda.synchronize()

@@ -349,3 +349,23 @@ def test_pow2_layer_against_float64_dense():
     assert moe.rel_rms_error(out, want) < 1e-4
     with pytest.raises(AssertionError):
         moe.moe_forward(x, logits, w13_q, w13_s * 1.5, w2_q, w2_s, top_k=2, pow2_scales=True)
+
+
+# ---- the bf16 RMS norm in front of the layer -----------------------------------------------------
+
+def test_rmsnorm_bf16_closed_form_and_golden():
+    from pathlib import Path
+    gen = torch.Generator().manual_seed(71)
+    x = (torch.randn(9, 384, generator=gen) * 3).bfloat16()
+    w = (1.0 + 0.2 * torch.randn(384, generator=gen)).bfloat16()
+    y = moe.rmsnorm_bf16(x, w)
+    assert y.dtype == torch.bfloat16
+    xd = x.double()
+    want = w.double() * xd / torch.sqrt(xd.pow(2).mean(-1, keepdim=True) + 1e-6)
+    assert ((y.double() - want).abs() <= want.abs() * 2.0 ** -7 + 1e-30).all()      # two bf16 roundings
+    z = np.load(Path(__file__).parent / 'golden' / 'rmsnorm_golden.npz')
+    got = moe.rmsnorm_bf16(torch.from_numpy(z['x']).bfloat16(), torch.from_numpy(z['weight']).bfloat16())
+    want = torch.from_numpy(z['y'])
+    # the module uses rsqrt, this restatement 1/sqrt: an fp32 ulp of the factor can move a value across a bf16 boundary
+    assert (got.float() == want).float().mean() >= 0.995
+    assert ((got.float() - want).abs() <= want.abs() * 2.0 ** -7).all()
