@@ -881,43 +881,70 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
     PHASE_TIMING_END(wave, lane);
 }
 
-// out[b, h, :] = sum_s w_s o_part[b, s, h, :],  w_s = exp2(lse_s - max) / sum; one workgroup of
-// 128 lanes per (b, h), 4 output columns per lane. PART is the type the split kernel stored:
-// float, or fp16 of O / scale with the per-head scale in scale_part.
-template <typename OUT, typename PART>
-__global__ __launch_bounds__(128) void sparse_mla_merge_kernel(const PART* __restrict__ o_part,
+// out[b, h, :] = sum_s w_s o_part[b, s, h, :],  w_s = exp2(lse_s - max) / sum. One wavefront per
+// (b, h), 8 output columns per lane, 4 heads per workgroup (grid x = n_heads / 4, y = request): the
+// rows of all splits are requested before the first is used. PART is the type the split kernel
+// stored: float, or fp16 of O / scale with the per-head scale in scale_part.
+// BATCH = splits whose rows a lane requests at once.
+template <typename OUT, typename PART, int BATCH>
+__global__ __launch_bounds__(256) void sparse_mla_merge_kernel(const PART* __restrict__ o_part,
                                                                const float* __restrict__ lse_part,
                                                                const float* __restrict__ scale_part,
                                                                OUT* __restrict__ out, int n_heads,
                                                                int n_splits) {
-    typedef PART partx4 __attribute__((ext_vector_type(4)));
-    const int h = blockIdx.x;
+    typedef PART partx8 __attribute__((ext_vector_type(8)));
+    typedef float floatx8 __attribute__((ext_vector_type(8)));
+    const int lane = threadIdx.x & 63;
+    const int h = blockIdx.x * 4 + (threadIdx.x >> 6);
     const int b = blockIdx.y;
     const size_t base = (size_t)b * n_splits * n_heads + h;
+    floatx8 o = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    float wsum = 0.f;
+    partx8 rows[BATCH];
+    auto load_rows = [&](int s0) {
+#pragma unroll
+        for (int j = 0; j < BATCH; ++j) {
+            // (splits past the end repeat the last one; their weight is 0)
+            const int s = s0 + j < n_splits ? s0 + j : n_splits - 1;
+            rows[j] = __builtin_nontemporal_load(
+                reinterpret_cast<const partx8*>(o_part + (base + (size_t)s * n_heads) * D_V) + lane);
+        }
+    };
+    // the first rows are requested before anything depends on the log-sum-exps
+    load_rows(0);
     float mx = -INFINITY;
     for (int s = 0; s < n_splits; ++s) mx = fmaxf(mx, lse_part[base + (size_t)s * n_heads]);
-    float wsum = 0.f;
-    floatx4 o = {0.f, 0.f, 0.f, 0.f};
-    if (mx > -INFINITY) {
-        for (int s = 0; s < n_splits; ++s) {
-            const float w = __builtin_amdgcn_exp2f(lse_part[base + (size_t)s * n_heads] - mx);
-            if (w > 0.f) {
-                const partx4 p = *reinterpret_cast<const partx4*>(
-                    o_part + (base + (size_t)s * n_heads) * D_V + threadIdx.x * 4);
-                floatx4 v = {(float)p.x, (float)p.y, (float)p.z, (float)p.w};
-                if constexpr (sizeof(PART) == 2) v *= scale_part[base + (size_t)s * n_heads];
-                o += v * w;
-                wsum += w;
+    for (int s0 = 0; s0 < n_splits; s0 += BATCH) {
+        if (s0 > 0) load_rows(s0);
+        float w[BATCH], sc[BATCH];
+#pragma unroll
+        for (int j = 0; j < BATCH; ++j) {
+            const int s = s0 + j < n_splits ? s0 + j : n_splits - 1;
+            const size_t row = base + (size_t)s * n_heads;
+            // (mx = -inf: every split is empty, all weights 0)
+            w[j] = s0 + j < n_splits && mx > -INFINITY ? __builtin_amdgcn_exp2f(lse_part[row] - mx) : 0.f;
+            sc[j] = 1.f;
+            if constexpr (sizeof(PART) == 2) sc[j] = scale_part[row];
+        }
+#pragma unroll
+        for (int j = 0; j < BATCH; ++j) {
+            if (w[j] > 0.f) {  // (a split without rows has weight 0 and is not looked at)
+                const float ws = w[j] * sc[j];  // sc is a power of two
+#pragma unroll
+                for (int i = 0; i < 8; ++i) o[i] += (float)rows[j][i] * ws;
+                wsum += w[j];
             }
         }
-        o *= 1.f / wsum;
     }
-    OUT* dst = out + ((size_t)b * n_heads + h) * D_V + threadIdx.x * 4;
+    if (wsum > 0.f) o *= 1.f / wsum;
+    OUT* dst = out + ((size_t)b * n_heads + h) * D_V + lane * 8;
     if constexpr (sizeof(OUT) == 4) {
-        *reinterpret_cast<floatx4*>(dst) = o;
+        reinterpret_cast<floatx4*>(dst)[0] = floatx4{o[0], o[1], o[2], o[3]};
+        reinterpret_cast<floatx4*>(dst)[1] = floatx4{o[4], o[5], o[6], o[7]};
     } else {
-        bf16x4 r = {(__bf16)o.x, (__bf16)o.y, (__bf16)o.z, (__bf16)o.w};
-        *reinterpret_cast<bf16x4*>(dst) = r;
+        const bf16x8 r = {(__bf16)o[0], (__bf16)o[1], (__bf16)o[2], (__bf16)o[3],
+                          (__bf16)o[4], (__bf16)o[5], (__bf16)o[6], (__bf16)o[7]};
+        *reinterpret_cast<bf16x8*>(dst) = r;
     }
 }
 
@@ -995,7 +1022,7 @@ void launch_sparse_mla(void* out, const void* q, const void* kv, const int* idx,
     const __bf16* qb = static_cast<const __bf16*>(q);
     const __bf16* kvb = static_cast<const __bf16*>(kv);
     const dim3 grid(splits, batch, head_groups);
-    const dim3 merge_grid(n_heads, batch);
+    const dim3 merge_grid(n_heads / 4, batch);
     bool half_parts = false;
     if (n_heads == 32) {
         sparse_mla_split_kernel<1><<<grid, 64, 0, stream>>>(qb, kvb, idx, o_part, lse_part, n_heads,
@@ -1015,22 +1042,30 @@ void launch_sparse_mla(void* out, const void* q, const void* kv, const int* idx,
             qb, kvb, idx, reinterpret_cast<_Float16*>(o_part), lse_part, scale_part, n_heads, n_kv_rows,
             topk, rows_per_split, scale_log2, kva);
     }
+    // rows requested at once per lane: as many as there are splits, up to 8
+#define MLA_MERGE(OUT_T, PART_T, PARTS, SCALES)                                                   \
+    if (splits <= 2)                                                                              \
+        sparse_mla_merge_kernel<OUT_T, PART_T, 2><<<merge_grid, 256, 0, stream>>>(                \
+            PARTS, lse_part, SCALES, static_cast<OUT_T*>(out), n_heads, splits);                  \
+    else if (splits <= 4)                                                                         \
+        sparse_mla_merge_kernel<OUT_T, PART_T, 4><<<merge_grid, 256, 0, stream>>>(                \
+            PARTS, lse_part, SCALES, static_cast<OUT_T*>(out), n_heads, splits);                  \
+    else                                                                                          \
+        sparse_mla_merge_kernel<OUT_T, PART_T, 8><<<merge_grid, 256, 0, stream>>>(                \
+            PARTS, lse_part, SCALES, static_cast<OUT_T*>(out), n_heads, splits);
     if (half_parts) {
         const _Float16* parts = reinterpret_cast<const _Float16*>(o_part);
         if (out_dtype == 0) {
-            sparse_mla_merge_kernel<__bf16, _Float16><<<merge_grid, 128, 0, stream>>>(
-                parts, lse_part, scale_part, static_cast<__bf16*>(out), n_heads, splits);
+            MLA_MERGE(__bf16, _Float16, parts, scale_part)
         } else {
-            sparse_mla_merge_kernel<float, _Float16><<<merge_grid, 128, 0, stream>>>(
-                parts, lse_part, scale_part, static_cast<float*>(out), n_heads, splits);
+            MLA_MERGE(float, _Float16, parts, scale_part)
         }
     } else if (out_dtype == 0) {
-        sparse_mla_merge_kernel<__bf16, float><<<merge_grid, 128, 0, stream>>>(
-            o_part, lse_part, nullptr, static_cast<__bf16*>(out), n_heads, splits);
+        MLA_MERGE(__bf16, float, o_part, nullptr)
     } else {
-        sparse_mla_merge_kernel<float, float><<<merge_grid, 128, 0, stream>>>(
-            o_part, lse_part, nullptr, static_cast<float*>(out), n_heads, splits);
+        MLA_MERGE(float, float, o_part, nullptr)
     }
+#undef MLA_MERGE
 }
 
 }  // namespace
