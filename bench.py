@@ -37,7 +37,8 @@ METRIC = "GB/s & % HBM peak (GDN/MoE/MLA decode); fp8 TFLOP/s % MFMA peak (MoE p
 # by the same counters read on a plain 512 MiB copy kernel (FETCH_SIZE x 1.99981, WRITE_SIZE x 1,
 # both in KiB); the counter summary is profiles/all_workloads_hbm_traffic_pmc.md.
 # None = not measured.
-MEASURED_TRAFFIC = {'gdn': 1085972770, 'moe_decode': 6664643628, 'mla': 223278459, 'index_scores': 553871480, 'moe_prefill': 11230161000}
+MEASURED_TRAFFIC = {'gdn': 1085972770, 'moe_decode': 6664643628, 'mla': 223326108, 'index_scores': 553871480,
+                    'index_scores_fp8': 289779791, 'moe_prefill': 11230161000}
 
 
 SETTLE_SECONDS = 0.05
@@ -355,6 +356,40 @@ def bench_index_scores(torch, capi, dev, steps, warmup, cpu_baseline):
     return res
 
 
+def bench_index_scores_fp8(torch, capi, dev, steps, warmup, cpu_baseline):
+    """The indexer scores over e4m3 index keys: the same shape as index_scores, 128 one-byte codes and one fp32
+    scale per cached position."""
+    from oracle import mla
+    B, Hi, N = 64, 64, 32768
+    gen = torch.Generator(device=dev).manual_seed(20263)
+    q = torch.randn(B, Hi, 128, device=dev, generator=gen).to(torch.float8_e4m3fn).view(torch.uint8)
+    # two key caches used in turn: one (277 MB with its scales) is about the size of the last-level cache
+    ks = [torch.randn(B, N, 128, device=dev, generator=gen).to(torch.float8_e4m3fn).view(torch.uint8) for _ in range(2)]
+    ss = [torch.rand(B, N, device=dev, generator=gen) + 0.5 for _ in range(2)]
+    w = torch.randn(B, Hi, device=dev, generator=gen) / 8
+    scores = torch.empty(B, N, device=dev)
+    sec = timed_launches(torch, lambda i: capi.mla_index_scores_fp8_launch(scores, q, ks[i % 2], ss[i % 2], w),
+                         steps, warmup)
+    work = B * N * 128 + B * N * 4 + B * N * 4 + B * Hi * 128 + B * Hi * 4
+    flops = 2 * B * Hi * N * 128
+    res = dict(
+        workload="indexer scores over e4m3 index keys: B=64, 64 index heads x 128, 32768 keys per request "
+                 "(128 codes + one fp32 scale each), seed 20263",
+        value=work / sec / 1e9, unit="GB/s", ms_per_step=sec * 1e3, dtype="e4m3", kernel="mla_index_scores_fp8_kernel",
+        roofline=dict(bound="hbm", achieved=work / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
+                      frac=work / sec / 1e9 / HBM_PEAK_GBS, traffic=MEASURED_TRAFFIC.get('index_scores_fp8')),
+        algorithmic_bytes=work, tflops=flops / sec / 1e12)
+    if cpu_baseline:
+        cores = len(os.sched_getaffinity(0))
+        torch.set_num_threads(cores)
+        nb = 2
+        hq, hk, hs, hw = q[:nb].cpu(), ks[0][:nb].cpu(), ss[0][:nb].cpu(), w[:nb].cpu()
+        csec = cpu_time(lambda: mla.index_scores_fp8(hq, hk, hs, hw))
+        res['cpu_baseline'] = dict(value=work / B * nb / csec / 1e9, unit="GB/s", cores=cores, kind="port",
+                                   sample="requests 0..1 (1/32 of the batch), eager PyTorch oracle in float64")
+    return res
+
+
 def bench_topk_select(torch, capi, dev, steps, warmup, cpu_baseline):
     """The selection in front of configs[3]: 2048 of 32768 index scores per request, 64 requests."""
     from oracle import mla
@@ -549,7 +584,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=20)
     ap.add_argument('--warmup', type=int, default=5)
-    ap.add_argument('--workloads', default='gdn,gdn_single,gdn_fused,gdn_fused_norm,conv1d,moe_decode,router_decode,index_scores,topk_select,mla,mla_paged,moe_prefill,router_prefill,rmsnorm_quant')
+    ap.add_argument('--workloads', default='gdn,gdn_single,gdn_fused,gdn_fused_norm,conv1d,moe_decode,router_decode,index_scores,index_scores_fp8,topk_select,mla,mla_paged,moe_prefill,router_prefill,rmsnorm_quant')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run 3 plain device copies of 536 870 912 bytes (a kernel of known traffic, '
@@ -592,6 +627,8 @@ def main():
             results[name] = bench_router(torch, capi, dev, args.steps, args.warmup, cpu, name == 'router_prefill')
         elif name == 'rmsnorm_quant':
             results[name] = bench_rmsnorm_quant(torch, capi, dev, args.steps, args.warmup, cpu)
+        elif name == 'index_scores_fp8':
+            results[name] = bench_index_scores_fp8(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'index_scores':
             results[name] = bench_index_scores(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'topk_select':

@@ -36,6 +36,9 @@ SIGNATURES = {
     'mla_index_scores_launcher': (None, [_P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_float, c_int, _P]),
     'mla_index_scores_paged_launcher': (None, [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int,
                                                c_float, c_int, _P]),
+    'mla_index_scores_fp8_launcher': (None, [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_float, c_int, _P]),
+    'mla_index_scores_fp8_paged_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int,
+                                                   c_int, c_float, c_int, _P]),
     'topk_select_launcher': (None, [_P, _P, _P, c_int, c_int, c_int, c_int, _P]),
     'moe_route_launcher': (None, [_P, _P, _P, c_int, c_int, c_int, c_int, _P]),
     'moe_router_logits_num_splits': (c_int, [c_int, c_int, c_int]),
@@ -331,6 +334,62 @@ def mla_index_scores_paged_launch(scores, q, k_pool, block_table, w, lengths=Non
         _ptr(lengths) if lengths is not None else c_void_p(None), B, Hi, n_pages, page, max_pages, D, float(scale),
         0, _stream(stream))
     check_status('mla_index_scores_paged_launcher')
+    return scores
+
+
+def _is_e4m3(t):
+    import torch
+    return t.dtype in (torch.uint8, torch.float8_e4m3fn)
+
+
+def mla_index_scores_fp8_launch(scores, q, k_cache, k_scale, w, lengths=None, scale=128 ** -0.5, stream=None):
+    """scores [B, N] fp32 <- k_scale[b,t] * sum_h w[b,h] * relu(scale * q[b,h] . k_cache[b,t]); -inf at
+    t >= lengths[b]. q [B, Hi, 128] and k_cache [B, N, 128] e4m3 codes (uint8 or float8_e4m3fn),
+    k_scale [B, N] fp32, w [B, Hi] fp32 (head weight times the scale of that head's q)."""
+    import torch
+    _device_contiguous(scores=scores, q=q, k_cache=k_cache, k_scale=k_scale, w=w)
+    B, Hi, D = q.shape
+    N = k_cache.shape[1]
+    _require(_is_e4m3(q) and _is_e4m3(k_cache) and k_scale.dtype == w.dtype == scores.dtype == torch.float32,
+             'mla_index_scores_fp8: q, k_cache e4m3 codes; k_scale, w, scores fp32')
+    _require(tuple(k_cache.shape) == (B, N, D) and tuple(k_scale.shape) == (B, N) and tuple(w.shape) == (B, Hi)
+             and tuple(scores.shape) == (B, N), 'mla_index_scores_fp8: shapes')
+    if lengths is not None:
+        _device_contiguous(lengths=lengths)
+        _require(lengths.dtype == torch.int32 and tuple(lengths.shape) == (B,),
+                 'mla_index_scores_fp8: lengths int32 [B]')
+    library().mla_index_scores_fp8_launcher(_ptr(scores), _ptr(q), _ptr(k_cache), _ptr(k_scale), _ptr(w),
+                                            _ptr(lengths) if lengths is not None else c_void_p(None), B, Hi, N, D,
+                                            float(scale), 0, _stream(stream))
+    check_status('mla_index_scores_fp8_launcher')
+    return scores
+
+
+def mla_index_scores_fp8_paged_launch(scores, q, k_pool, k_scale_pool, block_table, w, lengths=None,
+                                      scale=128 ** -0.5, stream=None):
+    """As ``mla_index_scores_fp8_launch`` over a paged key cache: k_pool [n_pages, page, 128] e4m3 codes,
+    k_scale_pool [n_pages, page] fp32, block_table [B, max_pages] int32; scores [B, max_pages * page]."""
+    import torch
+    _device_contiguous(scores=scores, q=q, k_pool=k_pool, k_scale_pool=k_scale_pool, block_table=block_table, w=w)
+    B, Hi, D = q.shape
+    n_pages, page = k_pool.shape[0], k_pool.shape[1]
+    max_pages = block_table.shape[1]
+    _require(_is_e4m3(q) and _is_e4m3(k_pool) and k_scale_pool.dtype == w.dtype == scores.dtype == torch.float32,
+             'mla_index_scores_fp8: q, k_pool e4m3 codes; k_scale_pool, w, scores fp32')
+    _require(block_table.dtype == torch.int32 and block_table.shape[0] == B,
+             'mla_index_scores_fp8: block_table int32 [B, P]')
+    _require(tuple(k_pool.shape) == (n_pages, page, D) and tuple(k_scale_pool.shape) == (n_pages, page)
+             and tuple(w.shape) == (B, Hi) and tuple(scores.shape) == (B, max_pages * page),
+             'mla_index_scores_fp8: shapes')
+    if lengths is not None:
+        _device_contiguous(lengths=lengths)
+        _require(lengths.dtype == torch.int32 and tuple(lengths.shape) == (B,),
+                 'mla_index_scores_fp8: lengths int32 [B]')
+    library().mla_index_scores_fp8_paged_launcher(
+        _ptr(scores), _ptr(q), _ptr(k_pool), _ptr(k_scale_pool), _ptr(block_table), _ptr(w),
+        _ptr(lengths) if lengths is not None else c_void_p(None), B, Hi, n_pages, page, max_pages, D, float(scale),
+        0, _stream(stream))
+    check_status('mla_index_scores_fp8_paged_launcher')
     return scores
 
 

@@ -189,6 +189,28 @@ void mla_index_scores_paged_launcher(float* scores, const void* q, const void* k
                                      int max_pages_per_request, int head_dim, float scale, int config,
                                      hipStream_t stream);
 
+/* Index scores over e4m3 index keys (the storage form of the indexer's key cache: 128 one-byte
+ * codes and one fp32 scale per position; caller-side neighbour, same launcher pattern
+ * agent_workdir/kernels/axpby.cu:12-20):
+ *   scores[b, t] = k_scale[b, t] * sum_h w[b, h] * max(0, scale * q[b, h, :] . k_cache[b, t, :])
+ *   q [batch, n_heads, 128] and k_cache [batch, n_rows, 128] OCP e4m3 codes (bias 7, no infinities),
+ *   k_scale [batch, n_rows] fp32 (key row = code * k_scale: what moe_quant_bf16_launcher writes for
+ *   rows of 128 values), w [batch, n_heads] fp32 = head weight * the scale that head's q was
+ *   quantised with. Masking, shapes and alignment as mla_index_scores_launcher. */
+void mla_index_scores_fp8_launcher(float* scores, const void* q, const void* k_cache,
+                                   const float* k_scale, const float* w, const int* lengths,
+                                   int batch, int n_heads, int n_rows, int head_dim, float scale,
+                                   int config, hipStream_t stream);
+
+/* The same over a paged e4m3 key cache: k_pool [n_pages, page_size, 128] codes and k_scale_pool
+ * [n_pages, page_size] fp32 shared by all requests; block table, scores and limits as
+ * mla_index_scores_paged_launcher. */
+void mla_index_scores_fp8_paged_launcher(float* scores, const void* q, const void* k_pool,
+                                         const float* k_scale_pool, const int* block_table,
+                                         const float* w, const int* lengths, int batch, int n_heads,
+                                         int n_pages, int page_size, int max_pages_per_request,
+                                         int head_dim, float scale, int config, hipStream_t stream);
+
 /* Top-k selection of index scores, the step that produces idx for the two launchers above
  * (caller-side neighbour; same launcher pattern agent_workdir/kernels/axpby.cu:12-20):
  *   idx_out [batch, k] int32: per request the indices of the k largest scores among the first

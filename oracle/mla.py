@@ -144,6 +144,37 @@ def index_scores(q, k_cache, w, lengths=None, scale=128 ** -0.5):
     return out
 
 
+def e4m3_to_float(codes):
+    """OCP e4m3 codes (uint8 tensor) -> fp32, from the bit fields: sign 1, exponent 4 (bias 7), mantissa 3;
+    exponent 0 is subnormal (mantissa / 8 * 2^-6), code 0x7f / 0xff is NaN, there are no infinities."""
+    c = codes.to(torch.int32)
+    sign = torch.where((c >> 7) == 1, -1.0, 1.0)
+    exp = (c >> 3) & 15
+    man = (c & 7).float()
+    normal = (1.0 + man / 8.0) * torch.pow(2.0, (exp - 7).float())
+    subnormal = man / 8.0 * 2.0 ** -6
+    val = torch.where(exp == 0, subnormal, normal)
+    val = torch.where((c & 0x7f) == 0x7f, torch.full_like(val, float('nan')), val)
+    return (sign * val).float()
+
+
+def index_scores_fp8(q_codes, k_codes, k_scale, w, lengths=None, scale=128 ** -0.5):
+    """Indexer scores over e4m3 keys: q_codes [B,Hi,d] and k_codes [B,N,d] uint8 e4m3 codes, k_scale [B,N]
+    fp32 (key = code * k_scale), w [B,Hi] fp32 (head weight times the scale of that head's q) ->
+    scores [B,N] fp32 = k_scale[b,t] * sum_h w[b,h] * relu(scale * q[b,h] . k[b,t]); -inf at positions >=
+    lengths[b]. The quantised form of ``index_scores`` (the third-party model file
+    transformers/models/deepseek_v32/modeling_deepseek_v32.py:203-212 states that its bf16 scoring stands
+    for an `fp8_index` kernel of the same formula); evaluated in float64."""
+    q = e4m3_to_float(q_codes).double()
+    k = e4m3_to_float(k_codes).double()
+    s = torch.relu(torch.einsum('bhd,bnd->bhn', q, k) * scale)
+    out = (torch.einsum('bh,bhn->bn', w.double(), s) * k_scale.double()).float()
+    if lengths is not None:
+        pos = torch.arange(k_codes.shape[1], device=out.device)[None, :]
+        out = out.masked_fill(pos >= lengths.to(out.device)[:, None].long(), float('-inf'))
+    return out
+
+
 def topk_select(scores, k, lengths=None):
     """Indices of the k largest scores per row among the first lengths[b] entries (all, if None):
     ties to the lower index, ascending index order, -1 where fewer than k candidates exist; NaN ranks

@@ -211,6 +211,50 @@ def test_index_scores_match_float64_loops_and_invariants():
     torch.testing.assert_close(mla.index_scores(q, k, 3 * w), 3 * mla.index_scores(q, k, w), rtol=1e-6, atol=1e-6)
 
 
+def test_index_scores_fp8_decode_loops_and_agreement_with_the_bf16_form():
+    from oracle import moe
+    # the decoder against an independent one (torch's cast), all 256 codes
+    codes = torch.arange(256, dtype=torch.uint8)
+    mine, theirs = mla.e4m3_to_float(codes), codes.view(torch.float8_e4m3fn).float()
+    assert torch.equal(torch.isnan(mine), torch.isnan(theirs))
+    assert torch.equal(mine[~torch.isnan(mine)], theirs[~torch.isnan(theirs)])
+    # plain float64 loops on a tiny case
+    gen = torch.Generator().manual_seed(35)
+    B, Hi, N, d = 2, 3, 7, 8
+    qc = torch.randint(0, 0x7f, (B, Hi, d), generator=gen).to(torch.uint8) | (torch.randint(0, 2, (B, Hi, d), generator=gen) << 7).to(torch.uint8)
+    kc = torch.randint(0, 0x7f, (B, N, d), generator=gen).to(torch.uint8) | (torch.randint(0, 2, (B, N, d), generator=gen) << 7).to(torch.uint8)
+    ks = torch.rand(B, N, generator=gen) + 0.5
+    w = torch.randn(B, Hi, generator=gen)
+    lengths = torch.tensor([7, 4], dtype=torch.int32)
+    got = mla.index_scores_fp8(qc, kc, ks, w, lengths, scale=2.0 ** -10)
+    qf, kf = qc.view(torch.float8_e4m3fn).double(), kc.view(torch.float8_e4m3fn).double()
+    for b in range(B):
+        for t in range(N):
+            if t >= int(lengths[b]):
+                assert got[b, t] == float('-inf')
+                continue
+            want = float(ks[b, t]) * sum(float(w[b, h]) * max(0.0, 2.0 ** -10 * sum(float(qf[b, h, j]) * float(kf[b, t, j]) for j in range(d)))
+                                         for h in range(Hi))
+            assert abs(float(got[b, t]) - want) <= 1e-6 * (1 + abs(want))
+    # the quantised form of the bf16 scores: on keys and queries that e4m3 holds exactly (scales a power of two)
+    # both oracles agree, and on quantised random inputs the scores stay within the quantisation error
+    B, Hi, N, d = 2, 8, 64, 128
+    q = torch.randn(B, Hi, d, generator=gen)
+    k = torch.randn(B, N, d, generator=gen)
+    w = torch.randn(B, Hi, generator=gen) * Hi ** -0.5
+    qq, qs = moe.quantize_groups(q.reshape(B * Hi, d), pow2=True)
+    kq, ks = moe.quantize_groups(k.reshape(B * N, d), pow2=True)
+    q_deq = (qq.float() * qs).reshape(B, Hi, d)
+    k_deq = (kq.float() * ks).reshape(B, N, d)
+    assert torch.equal(q_deq.bfloat16().float(), q_deq) and torch.equal(k_deq.bfloat16().float(), k_deq)
+    fp8 = mla.index_scores_fp8(qq.view(torch.uint8).reshape(B, Hi, d), kq.view(torch.uint8).reshape(B, N, d),
+                               ks.reshape(B, N), w * qs.reshape(B, Hi))
+    torch.testing.assert_close(fp8, mla.index_scores(q_deq.bfloat16(), k_deq.bfloat16(), w), rtol=1e-5, atol=1e-5)
+    exact = mla.index_scores(q.bfloat16(), k.bfloat16(), w)
+    assert mla.rel_rms_error(fp8, exact) < 0.5      # (e4m3 keeps 3 mantissa bits: the scores move by a few per cent)
+    assert torch.nn.functional.cosine_similarity(fp8.flatten(), exact.flatten(), dim=0) > 0.99
+
+
 def test_index_scores_select_what_the_third_party_indexer_selects():
     from pathlib import Path
     z = np.load(Path(__file__).parent / 'golden' / 'indexer_golden.npz')
