@@ -186,3 +186,50 @@ def test_moe_layer_with_shared_expert_in_a_graph(capi, dev):
         torch.cuda.synchronize()
         assert torch.equal(out, eager)
         eager_noise(dev)
+
+
+def test_fp8_indexer_chain_in_a_graph(capi, dev):
+    # the new token's index key is quantised into the e4m3 key cache, then scores -> selection -> attention
+    gen = torch.Generator().manual_seed(19)
+    B, H, Hi, N, k = 2, 128, 64, 1024, 256
+    q, kv, _ = mla.mla_make_inputs(B, H, N, k, generator=gen)
+    q, kv = q.to(dev), kv.to(dev)
+    keys = (torch.randn(B, N, 128, generator=gen) * 2).bfloat16().to(dev)
+    codes = torch.zeros(B, N, 128, dtype=torch.uint8, device=dev)
+    kscale = torch.ones(B, N, device=dev)
+    capi.moe_quant_bf16_launch(codes.view(B * N, 128), kscale.view(B * N, 1), keys.view(B * N, 128))
+    q_idx = torch.randn(B, Hi, 128, generator=gen).to(torch.float8_e4m3fn).view(torch.uint8).to(dev)
+    w = (torch.randn(B, Hi, generator=gen) / 8).to(dev)
+    lengths = torch.tensor([N, 700], dtype=torch.int32, device=dev)
+    new_key = torch.empty(B, 128, dtype=torch.bfloat16, device=dev)
+    new_codes = torch.empty(B, 128, dtype=torch.uint8, device=dev)
+    new_scale = torch.empty(B, 1, device=dev)
+    ws = torch.empty(capi.sparse_mla_workspace_bytes(B, H, k), dtype=torch.uint8, device=dev)
+
+    def step(scores, idx, out, ws):
+        capi.moe_quant_bf16_launch(new_codes, new_scale, new_key)
+        codes[:, 5].copy_(new_codes)                         # position 5 of every request takes the new key
+        kscale[:, 5].copy_(new_scale[:, 0])
+        capi.mla_index_scores_fp8_launch(scores, q_idx, codes, kscale, w, lengths)
+        capi.topk_select_launch(idx, scores, lengths)
+        capi.sparse_mla_decode_launch(out, q, kv, idx, ws)
+
+    sc_g, sc_e = (torch.empty(B, N, device=dev) for _ in range(2))
+    idx_g, idx_e = (torch.empty(B, k, dtype=torch.int32, device=dev) for _ in range(2))
+    out_g, out_e = (torch.empty(B, H, 512, dtype=torch.bfloat16, device=dev) for _ in range(2))
+    new_key.copy_(torch.randn(B, 128, device=dev))
+    graph = capture(lambda: step(sc_g, idx_g, out_g, ws))
+    ws_e = torch.empty_like(ws)
+    for r in range(3):
+        new_key.copy_(torch.randn(B, 128, device=dev) * (r + 1))
+        out_g.fill_(float('nan'))
+        graph.replay()
+        torch.cuda.synchronize()
+        step(sc_e, idx_e, out_e, ws_e)
+        torch.cuda.synchronize()
+        assert torch.equal(sc_g, sc_e) and torch.equal(idx_g, idx_e) and torch.equal(out_g, out_e)
+        want = mla.index_scores_fp8(q_idx.cpu(), codes.cpu(), kscale.cpu(), w.cpu(), lengths.cpu())
+        live = torch.isfinite(want)
+        torch.testing.assert_close(sc_g.cpu()[live], want[live], rtol=2e-3, atol=2e-3)
+        assert torch.equal(idx_g.cpu(), mla.topk_select(sc_g.cpu(), k, lengths.cpu()))
+        eager_noise(dev)
