@@ -604,12 +604,16 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
     // i.e. the two wavefronts of a pair alternate 32-element slices of d. The wait for Q also
     // waits for the two tiles issued above (loads return in order), which the loop needs anyway.
     // (requested here, behind the indices: Q does not depend on them, so its latency overlaps theirs)
-    bf16x8 qreg[HALF_K_STEPS];
+    // The loads take the wavefront's 64 bytes of every 128-byte line of Q from 16 rows per instruction
+    // (lane -> row 16*(l&1) + lane/4, 16-byte piece lane%4 of line l/2: 16 line requests instead of the 32 that
+    // loading the operand layout directly needs); the operand layout is made below through LDS.
+    uintx4 qraw[HALF_K_STEPS];
     {
-        const __bf16* qrow = q + ((size_t)b * n_heads + head0 + (lane & 31)) * D_QK + 8 * half + 32 * dh;
+        const char* qsrc = reinterpret_cast<const char*>(q + ((size_t)b * n_heads + head0) * D_QK) +
+                           (size_t)(lane >> 2) * ROW_BYTES + 64 * dh + 16 * (lane & 3);
 #pragma unroll
         for (int l = 0; l < HALF_K_STEPS; ++l) {
-            qreg[l] = *reinterpret_cast<const bf16x8*>(qrow + 64 * (l >> 1) + 16 * (l & 1));
+            qraw[l] = *reinterpret_cast<const uintx4*>(qsrc + (size_t)(16 * (l & 1)) * ROW_BYTES + 128 * (l >> 1));
         }
     }
     if (kva.block_table != nullptr) {
@@ -656,6 +660,27 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
     }
     PHASE_MARK(9);  // first gather issue
 
+    // Q into operand layout (lane = head lane%32, 16-byte piece 2*(l&1) + half of line l/2), one line of the
+    // 32 heads at a time through this wavefront's exchange buffer, which the loop does not use yet: rows of
+    // 64 bytes, piece p of row r at slot p ^ ((r >> 2) & 3) so that the 16 rows a read serves per cycle hit
+    // 16 different bank groups. No barrier: the LDS operations of a wavefront execute in order.
+    bf16x8 qreg[HALF_K_STEPS];
+    {
+        uintx4* stage = reinterpret_cast<uintx4*>(&s_xchg[wave][0]);
+        const int r = lane & 31;
+#pragma unroll
+        for (int j = 0; j < HALF_K_STEPS / 2; ++j) {
+#pragma unroll
+            for (int sl = 0; sl < 2; ++sl) {
+                const int wr = 16 * sl + (lane >> 2);
+                stage[wr * 4 + ((lane & 3) ^ ((wr >> 2) & 3))] = qraw[2 * j + sl];
+            }
+#pragma unroll
+            for (int sl = 0; sl < 2; ++sl) {
+                qreg[2 * j + sl] = __builtin_bit_cast(bf16x8, stage[r * 4 + ((2 * sl + half) ^ ((r >> 2) & 3))]);
+            }
+        }
+    }
 #pragma unroll
     for (int ks = 0; ks < HALF_K_STEPS; ++ks) asm volatile("" : "+v"(qreg[ks]));
     PHASE_MARK(8);  // wait for Q
