@@ -801,10 +801,17 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
         float psum = 0.f;
         bf16x8 p[2];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const __bf16 e = (__bf16)__builtin_amdgcn_exp2f(s[i] - m_use);
-            p[i / 8][i % 8] = e;
-            psum += (float)e;
+        for (int i = 0; i < 16; ++i) p[i / 8][i % 8] = (__bf16)__builtin_amdgcn_exp2f(s[i] - m_use);
+        // the normaliser sums the probabilities as rounded (see process_tile); v_dot2c_f32_bf16 adds two of
+        // them per instruction
+        {
+            typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+            const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+#pragma unroll
+            for (int i = 0; i < 16; i += 2) {
+                const bf16x2 pair = {p[i / 8][i % 8], p[i / 8][i % 8 + 1]};
+                psum = __builtin_amdgcn_fdot2_f32_bf16(pair, ones, psum, false);
+            }
         }
         st.l = st.l * alpha + psum;
         if (__builtin_amdgcn_ballot_w64(rescale) != 0) {
