@@ -28,6 +28,40 @@ __device__ __forceinline__ float key_logit(unsigned long long key) {
     return __uint_as_float((u & 0x80000000u) ? (u & 0x7fffffffu) : ~u);
 }
 
+// Maximum of a 32-bit unsigned value over the wavefront, returned as the same value in every lane. The
+// running maximum inside each row of 16 lanes goes through the DPP row shifts of the vector ALU, and the
+// last lanes of the four rows are read as scalars: no LDS crossbar, which the __shfl exchanges use and
+// which made a dependent chain of them cost about 100 cycles per step.
+__device__ __forceinline__ unsigned wave_max_u32(unsigned v) {
+    // dpp control 0x110 + n = row_shr:n; lanes without a source lane take `old` = 0, the identity
+#define ROW_SHR_MAX(n)                                                                              \
+    {                                                                                               \
+        const unsigned o = (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x110 + (n), 0xf, 0xf, false); \
+        v = o > v ? o : v;                                                                          \
+    }
+    ROW_SHR_MAX(1)
+    ROW_SHR_MAX(2)
+    ROW_SHR_MAX(4)
+    ROW_SHR_MAX(8)
+#undef ROW_SHR_MAX
+    const unsigned r0 = (unsigned)__builtin_amdgcn_readlane((int)v, 15);
+    const unsigned r1 = (unsigned)__builtin_amdgcn_readlane((int)v, 31);
+    const unsigned r2 = (unsigned)__builtin_amdgcn_readlane((int)v, 47);
+    const unsigned r3 = (unsigned)__builtin_amdgcn_readlane((int)v, 63);
+    const unsigned a = r0 > r1 ? r0 : r1;
+    const unsigned b = r2 > r3 ? r2 : r3;
+    return a > b ? a : b;
+}
+
+// maximum of the 64-bit rank keys of a wavefront: the largest upper half, then the largest lower half
+// among the lanes that hold it
+__device__ __forceinline__ unsigned long long wave_max_key(unsigned long long key) {
+    const unsigned hi = (unsigned)(key >> 32);
+    const unsigned hi_max = wave_max_u32(hi);
+    const unsigned lo_max = wave_max_u32(hi == hi_max ? (unsigned)key : 0u);
+    return ((unsigned long long)hi_max << 32) | lo_max;
+}
+
 template <int PER_LANE>
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits,
                                                         int* __restrict__ ids,
@@ -52,11 +86,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
         unsigned long long best = 0ull;
 #pragma unroll
         for (int j = 0; j < PER_LANE; ++j) best = key[j] > best ? key[j] : best;
-#pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) {
-            const unsigned long long other = __shfl_xor(best, off);
-            best = other > best ? other : best;
-        }
+        best = wave_max_key(best);
         const int id = 0x7fffffff - (int)(unsigned)(best & 0xffffffffull);
 #pragma unroll
         for (int j = 0; j < PER_LANE; ++j) {
@@ -154,11 +184,7 @@ __global__ __launch_bounds__(256) void moe_route_grouped_kernel(
         unsigned long long best = 0ull;
 #pragma unroll
         for (int j = 0; j < PER_LANE; ++j) best = key[j] > best ? key[j] : best;
-#pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) {
-            const unsigned long long other = __shfl_xor(best, off);
-            best = other > best ? other : best;
-        }
+        best = wave_max_key(best);
         const int id = 0x7fffffff - (int)(unsigned)(best & 0xffffffffull);
 #pragma unroll
         for (int j = 0; j < PER_LANE; ++j) {
@@ -368,8 +394,6 @@ __global__ __launch_bounds__(1024) void moe_route_sort_small_kernel(
     const int pairs = tokens * slots;
     for (int e = threadIdx.x; e <= sorted_experts; e += 1024) s_count[e] = 0;
     for (int i = threadIdx.x; i < 16 * (512 + 1); i += 1024) (&s_wave_count[0][0])[i] = 0;
-    // (The 8 arg-max rounds of the 64 tokens are bound by the cross-lane exchanges of the 16 wavefronts,
-    // which all go through the one LDS crossbar of this CU: about 2.3 us per round.)
     for (int t = wave; t < tokens; t += 16) {
         unsigned long long key[PER_LANE];
 #pragma unroll
@@ -383,11 +407,7 @@ __global__ __launch_bounds__(1024) void moe_route_sort_small_kernel(
             unsigned long long best = 0ull;
 #pragma unroll
             for (int j = 0; j < PER_LANE; ++j) best = key[j] > best ? key[j] : best;
-#pragma unroll
-            for (int off = 32; off >= 1; off >>= 1) {
-                const unsigned long long other = __shfl_xor(best, off);
-                best = other > best ? other : best;
-            }
+            best = wave_max_key(best);
             const int id = 0x7fffffff - (int)(unsigned)(best & 0xffffffffull);
 #pragma unroll
             for (int j = 0; j < PER_LANE; ++j) {
