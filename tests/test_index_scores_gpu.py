@@ -224,9 +224,10 @@ def test_fp8_keys_from_the_quantiser_and_selection(capi, dev):
     assert overlap > 0.9
 
 
-def test_fp8_paged_key_cache(capi, dev):
-    gen = torch.Generator().manual_seed(31)
-    B, Hi, N, page = 3, 64, 1024, 64
+@pytest.mark.parametrize('page', [16, 64, 256])
+def test_fp8_paged_key_cache(capi, dev, page):
+    gen = torch.Generator().manual_seed(31 + page)
+    B, Hi, N = 3, 64, 1024
     qc, kc, ks, w = make_fp8(B, Hi, N, 32)
     lengths = torch.tensor([N, 700, 333], dtype=torch.int32)
     want = run_fp8(capi, dev, qc, kc, ks, w, lengths)
@@ -239,7 +240,7 @@ def test_fp8_paged_key_cache(capi, dev):
     s_pool[order] = ks.reshape(B * per_req, page)
     table = order.reshape(B, per_req).int()
     table[1, 2] = -1
-    want[1, 128:192] = float('-inf')
+    want[1, 2 * page:3 * page] = float('-inf')
     scores = torch.full((B, N), float('nan'), device=dev)
     capi.mla_index_scores_fp8_paged_launch(scores, qc.to(dev), k_pool.to(dev), s_pool.to(dev), table.to(dev), w.to(dev),
                                            lengths.to(dev))
