@@ -458,6 +458,30 @@ def bench_mla(torch, capi, dev, steps, warmup, cpu_baseline, paged=False):
     return res
 
 
+def bench_mla_fp8_cache(torch, capi, dev, steps, warmup, cpu_baseline):
+    """configs[3] over the e4m3 storage form of the latent cache (656-byte rows): gather + dequantise of the
+    selected rows into the workspace, then the bf16 decode kernels on that block."""
+    B, H, N, topk = 64, 128, 32768, 2048
+    gen = torch.Generator(device=dev).manual_seed(20253)
+    q = torch.randn(B, H, 576, device=dev, generator=gen).bfloat16()
+    cache = torch.empty(B, N, 656, dtype=torch.uint8, device=dev)
+    for b0 in range(0, B, 8):
+        capi.mla_latent_quant_launch(cache[b0:b0 + 8], torch.randn(8, N, 576, device=dev, generator=gen).bfloat16())
+    idxs = [torch.stack([torch.randperm(N, device=dev, generator=gen)[:topk] for _ in range(B)]).int()
+            for _ in range(4)]
+    out = torch.empty(B, H, 512, device=dev, dtype=torch.bfloat16)
+    ws = torch.empty(capi.sparse_mla_fp8_workspace_bytes(B, H, topk), dtype=torch.uint8, device=dev)
+    sec = timed_launches(torch, lambda i: capi.sparse_mla_decode_fp8_launch(out, q, cache, idxs[i % 4], ws), steps, warmup)
+    work = B * topk * 656
+    return dict(
+        workload="configs[3] over an e4m3 latent cache: B=64, 128 heads, top-k 2048 of 32768 rows of 656 bytes (512 "
+                 "codes, 4 scales, 64 bf16 rope values), seed 20253 (gather + dequantise, split kernel, merge per step)",
+        value=work / sec / 1e9, unit="GB/s", ms_per_step=sec * 1e3, dtype="bf16", kernel="sparse_mla_split8_kernel",
+        roofline=dict(bound="hbm", achieved=work / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
+                      frac=work / sec / 1e9 / HBM_PEAK_GBS, traffic=None),
+        algorithmic_bytes=work)
+
+
 def make_moe(torch, dev, tokens, biased):
     """The workload's tensors. The weight buffers hold one more expert behind the 256 routed ones (the shared
     expert of the `with_shared_expert` timings, seed 20258); the routed experts are views of the first 256."""
@@ -584,7 +608,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=20)
     ap.add_argument('--warmup', type=int, default=5)
-    ap.add_argument('--workloads', default='gdn,gdn_single,gdn_fused,gdn_fused_norm,conv1d,moe_decode,router_decode,index_scores,index_scores_fp8,topk_select,mla,mla_paged,moe_prefill,router_prefill,rmsnorm_quant')
+    ap.add_argument('--workloads', default='gdn,gdn_single,gdn_fused,gdn_fused_norm,conv1d,moe_decode,router_decode,index_scores,index_scores_fp8,topk_select,mla,mla_paged,mla_fp8_cache,moe_prefill,router_prefill,rmsnorm_quant')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run 3 plain device copies of 536 870 912 bytes (a kernel of known traffic, '
@@ -635,6 +659,8 @@ def main():
             results[name] = bench_topk_select(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'mla':
             results[name] = bench_mla(torch, capi, dev, args.steps, args.warmup, cpu)
+        elif name == 'mla_fp8_cache':
+            results[name] = bench_mla_fp8_cache(torch, capi, dev, args.steps, args.warmup, cpu)
         elif name == 'mla_paged':
             results[name] = bench_mla(torch, capi, dev, args.steps, args.warmup, cpu, paged=True)
         elif name == 'moe_decode':

@@ -8,7 +8,7 @@ every output and scratch buffer is allocated by the caller, as the launcher ABI 
 """
 
 import ctypes
-from ctypes import c_float, c_int, c_size_t, c_void_p
+from ctypes import c_float, c_int, c_long, c_size_t, c_void_p
 
 from . import CAPI_LIBRARY
 
@@ -33,6 +33,10 @@ SIGNATURES = {
                                                 _P]),
     'sparse_mla_decode_num_splits': (c_int, [c_int, c_int, c_int, c_int]),
     'sparse_mla_decode_workspace_bytes': (c_size_t, [c_int, c_int, c_int, c_int]),
+    'mla_latent_quant_launcher': (None, [_P, _P, c_long, c_int, _P]),
+    'sparse_mla_decode_fp8_workspace_bytes': (c_size_t, [c_int, c_int, c_int, c_int]),
+    'sparse_mla_decode_fp8_launcher': (None, [_P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int,
+                                              c_float, c_int, c_int, _P]),
     'mla_index_scores_launcher': (None, [_P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_float, c_int, _P]),
     'mla_index_scores_paged_launcher': (None, [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int,
                                                c_float, c_int, _P]),
@@ -289,6 +293,50 @@ def sparse_mla_decode_paged_launch(out, q, kv_pool, block_table, idx, workspace,
         page_size, max_pages, topk, d_qk, d_v, float(sm_scale),
         0 if out.dtype == torch.bfloat16 else 1, config, _stream(stream))
     check_status('sparse_mla_decode_paged_launcher')
+    return out
+
+
+LATENT_ROW_BYTES = 656
+
+
+def mla_latent_quant_launch(cache, kv, config=0, stream=None):
+    """cache [..., 656] uint8 <- the e4m3 storage form of the latent rows kv [..., 576] bf16 (512 codes, 4 fp32
+    block scales, 64 bf16 rope values per row). config 32: power-of-two scales."""
+    import torch
+    _device_contiguous(cache=cache, kv=kv)
+    _require(kv.dtype == torch.bfloat16 and cache.dtype == torch.uint8, 'mla_latent_quant: kv bf16, cache uint8')
+    _require(kv.shape[-1] == 576 and cache.shape[-1] == LATENT_ROW_BYTES and tuple(kv.shape[:-1]) == tuple(cache.shape[:-1]),
+             'mla_latent_quant: kv [..., 576], cache [..., 656]')
+    rows = kv.numel() // 576
+    library().mla_latent_quant_launcher(_ptr(cache), _ptr(kv), rows, config, _stream(stream))
+    check_status('mla_latent_quant_launcher')
+    return cache
+
+
+def sparse_mla_fp8_workspace_bytes(batch, n_heads, topk, config=0):
+    return int(library().sparse_mla_decode_fp8_workspace_bytes(batch, n_heads, topk, config))
+
+
+def sparse_mla_decode_fp8_launch(out, q, kv_fp8, idx, workspace, sm_scale=192 ** -0.5, config=0, stream=None):
+    """As ``sparse_mla_decode_launch`` over kv_fp8 [B, N, 656] uint8, the e4m3 storage form of the latent cache.
+    ``workspace``: at least ``sparse_mla_fp8_workspace_bytes`` bytes."""
+    import torch
+    _device_contiguous(out=out, q=q, kv_fp8=kv_fp8, idx=idx, workspace=workspace)
+    B, H, d_qk = q.shape
+    N = kv_fp8.shape[1]
+    topk = idx.shape[1]
+    d_v = out.shape[2]
+    _require(q.dtype == torch.bfloat16 and kv_fp8.dtype == torch.uint8, 'sparse_mla_fp8: q bf16, kv_fp8 uint8')
+    _require(out.dtype in (torch.bfloat16, torch.float32), 'sparse_mla_fp8: out must be bf16 or fp32')
+    _require(idx.dtype == torch.int32, 'sparse_mla_fp8: idx must be int32')
+    _require(tuple(kv_fp8.shape) == (B, N, LATENT_ROW_BYTES) and tuple(idx.shape) == (B, topk),
+             'sparse_mla_fp8: kv_fp8 [B, N, 656], idx [B, topk]')
+    _require(tuple(out.shape) == (B, H, d_v), 'sparse_mla_fp8: out shape')
+    _require(workspace.dtype == torch.uint8, 'sparse_mla_fp8: workspace must be uint8')
+    library().sparse_mla_decode_fp8_launcher(
+        _ptr(out), _ptr(q), _ptr(kv_fp8), _ptr(idx), _ptr(workspace), workspace.numel(), B, H, N, topk, d_qk, d_v,
+        float(sm_scale), 0 if out.dtype == torch.bfloat16 else 1, config, _stream(stream))
+    check_status('sparse_mla_decode_fp8_launcher')
     return out
 
 

@@ -166,6 +166,26 @@ int sparse_mla_decode_num_splits(int batch, int n_heads, int topk, int config);
 /* Bytes of workspace sparse_mla_decode_launcher needs for these sizes and this config. */
 size_t sparse_mla_decode_workspace_bytes(int batch, int n_heads, int topk, int config);
 
+/* e4m3 storage form of the latent cache (caller-side neighbour of sparse_mla_decode_launcher; same launcher
+ * pattern agent_workdir/kernels/axpby.cu:12-20). A row is 656 bytes: 512 e4m3 codes of the latent values,
+ * 4 fp32 scales (scale i: values [128*i, 128*i+128), value = code * scale), then the 64 rope values as bf16.
+ * mla_latent_quant_launcher writes such rows from bf16 rows kv [rows, 576]: scale = amax / 448 per block of
+ * 128, or with config bit 32 the smallest power of two that is at least that. cache and kv 16-byte aligned. */
+void mla_latent_quant_launcher(void* cache, const void* kv, long rows, int config, hipStream_t stream);
+
+/* Workspace bytes of sparse_mla_decode_fp8_launcher: the workspace of sparse_mla_decode_launcher plus a
+ * block [batch, topk, 576] bf16 of dequantised selected rows and its index list. */
+size_t sparse_mla_decode_fp8_workspace_bytes(int batch, int n_heads, int topk, int config);
+
+/* sparse_mla_decode_launcher over kv_fp8 [batch, n_kv_rows, 656] bytes in the form above: the selected rows
+ * are gathered and dequantised (code * scale in fp32, rounded to nearest-even bf16) into the workspace, then
+ * attended as by sparse_mla_decode_launcher; the result equals that launcher's on the dequantised cache
+ * bit for bit. Other arguments, limits and config as there. */
+void sparse_mla_decode_fp8_launcher(void* out, const void* q, const void* kv_fp8, const int* idx,
+                                    void* workspace, size_t workspace_bytes, int batch, int n_heads,
+                                    int n_kv_rows, int topk, int d_qk, int d_v, float sm_scale,
+                                    int out_dtype, int config, hipStream_t stream);
+
 /* Index scores of the sparse-attention indexer, decode step (caller-side neighbour of the top-k
  * selection below; same launcher pattern agent_workdir/kernels/axpby.cu:12-20):
  *   scores[b, t] = sum_h w[b, h] * max(0, scale * q[b, h, :] . k_cache[b, t, :])  for t < lengths[b]

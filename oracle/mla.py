@@ -144,6 +144,54 @@ def index_scores(q, k_cache, w, lengths=None, scale=128 ** -0.5):
     return out
 
 
+LATENT_ROW_BYTES = 656      # 512 e4m3 codes + 4 fp32 scales + 64 bf16 rope values
+
+
+def latent_quantize(kv, pow2=False):
+    """The e4m3 storage form of latent cache rows: kv [..., 576] bf16 -> uint8 [..., 656]. Bytes [0,512): codes of
+    the 512 latent values, quantised per block of 128 with scale = amax/448 (``pow2``: the smallest power of two that
+    is at least that), exactly as the MoE activation quantiser (oracle.moe.quantize_groups); bytes [512,528): the 4
+    scales, little-endian fp32; bytes [528,656): the 64 rope values as bf16, unchanged. The layout is the one
+    third-party sparse-attention decoders document for an fp8 latent cache; no file of theirs is available here,
+    so it is pinned by its own description only (parity unpinned against a third-party implementation)."""
+    from oracle import moe
+    lead = kv.shape[:-1]
+    flat = kv.reshape(-1, 576)
+    codes, scales = moe.quantize_groups(flat[:, :512].float(), pow2=pow2)
+    out = torch.empty(flat.shape[0], LATENT_ROW_BYTES, dtype=torch.uint8)
+    out[:, :512] = codes.view(torch.uint8)
+    out[:, 512:528] = scales.contiguous().view(torch.uint8).reshape(-1, 16)
+    out[:, 528:] = flat[:, 512:].contiguous().view(torch.uint8).reshape(-1, 128)
+    return out.reshape(*lead, LATENT_ROW_BYTES)
+
+
+def latent_dequantize(cache):
+    """uint8 [..., 656] -> bf16 [..., 576]: code * scale in fp32, rounded to nearest-even bf16; rope as stored."""
+    lead = cache.shape[:-1]
+    flat = cache.reshape(-1, LATENT_ROW_BYTES)
+    codes = e4m3_to_float(flat[:, :512])
+    scales = flat[:, 512:528].contiguous().view(torch.float32)             # [rows, 4]
+    latent = (codes.reshape(-1, 4, 128) * scales[:, :, None]).reshape(-1, 512).bfloat16()
+    rope = flat[:, 528:].contiguous().view(torch.bfloat16)
+    return torch.cat([latent, rope], dim=1).reshape(*lead, 576)
+
+
+def latent_dequantize_device(cache):
+    """latent_dequantize on whatever device the cache is on (the codes through torch's own e4m3 cast)."""
+    lead = cache.shape[:-1]
+    flat = cache.reshape(-1, LATENT_ROW_BYTES)
+    codes = flat[:, :512].contiguous().view(torch.float8_e4m3fn).float()
+    scales = flat[:, 512:528].contiguous().view(torch.float32)
+    latent = (codes.reshape(-1, 4, 128) * scales[:, :, None]).reshape(-1, 512).bfloat16()
+    rope = flat[:, 528:].contiguous().view(torch.bfloat16)
+    return torch.cat([latent, rope], dim=1).reshape(*lead, 576)
+
+
+def sparse_mla_decode_fp8(q, cache, idx, **kwargs):
+    """sparse_mla_decode over a cache in the 656-byte form: attention over the dequantised rows."""
+    return sparse_mla_decode(q, latent_dequantize(cache.cpu()), idx, **kwargs)
+
+
 def e4m3_to_float(codes):
     """OCP e4m3 codes (uint8 tensor) -> fp32, from the bit fields: sign 1, exponent 4 (bias 7), mantissa 3;
     exponent 0 is subnormal (mantissa / 8 * 2^-6), code 0x7f / 0xff is NaN, there are no infinities."""

@@ -262,3 +262,50 @@ def test_index_scores_select_what_the_third_party_indexer_selects():
     scores = mla.index_scores(q, k, w, scale=float(z['scale'][0]))
     idx = mla.topk_select(scores, z['topk'].shape[1])
     np.testing.assert_array_equal(idx.numpy(), z['topk'])
+
+
+# ---- e4m3 storage form of the latent cache ---------------------------------------------------------------
+
+def test_latent_cache_layout_round_trip_and_error_bound():
+    import struct
+    gen = torch.Generator().manual_seed(41)
+    kv = (torch.randn(5, 576, generator=gen) * 3).bfloat16()
+    kv[1, 128:256] = 0
+    for pow2 in (False, True):
+        cache = mla.latent_quantize(kv, pow2=pow2)
+        assert cache.shape == (5, mla.LATENT_ROW_BYTES) and cache.dtype == torch.uint8
+        # the layout, field by field, with plain loops
+        for r in range(5):
+            row = bytes(cache[r].tolist())
+            scales = struct.unpack('<4f', row[512:528])
+            for blk in range(4):
+                vals = kv[r, 128 * blk:128 * blk + 128].float()
+                amax = max(float(vals.abs().max()), 1e-12)
+                if pow2:
+                    assert scales[blk] >= amax / 448 * (1 - 1e-6) and scales[blk] / 2 < amax / 448
+                    m, _ = np.frexp(scales[blk])
+                    assert m == 0.5
+                else:
+                    assert abs(scales[blk] - amax / 448) <= 1e-6 * amax / 448
+                for j in (0, 17, 127):
+                    code = torch.tensor([row[128 * blk + j]], dtype=torch.uint8).view(torch.float8_e4m3fn).float().item()
+                    want = float(vals[j]) / scales[blk]
+                    assert abs(code - want) <= max(abs(want) * 2.0 ** -4, 2.0 ** -10)
+            rope = torch.tensor(list(row[528:]), dtype=torch.uint8).view(torch.bfloat16)
+            assert torch.equal(rope, kv[r, 512:])
+        deq = mla.latent_dequantize(cache)
+        assert torch.equal(deq, mla.latent_dequantize_device(cache))
+        assert torch.equal(deq[:, 512:], kv[:, 512:])
+        blocks = kv[:, :512].float().reshape(5, 4, 128)
+        bound = blocks.abs().amax(dim=-1, keepdim=True) * (2.0 ** -4 + 2.0 ** -8) * (2 if pow2 else 1)
+        assert ((deq[:, :512].float().reshape(5, 4, 128) - blocks).abs() <= bound + 1e-30).all()
+    # values e4m3 holds exactly with a power-of-two block maximum survive the round trip unchanged
+    exact = torch.zeros(2, 576)
+    exact[:, :512] = torch.randint(-8, 9, (2, 512), generator=gen).float() * 0.25
+    exact[:, 0:512:128] = 448 * 2.0 ** -6
+    exact = exact.bfloat16()
+    assert torch.equal(mla.latent_dequantize(mla.latent_quantize(exact, pow2=True)), exact)
+    # attention over the fp8 cache = attention over the dequantised rows
+    q, kv2, idx = mla.mla_make_inputs(2, 4, 64, 16, generator=gen)
+    cache = mla.latent_quantize(kv2)
+    assert torch.equal(mla.sparse_mla_decode_fp8(q, cache, idx), mla.sparse_mla_decode(q, mla.latent_dequantize(cache), idx))
