@@ -31,6 +31,9 @@ SIGNATURES = {
     'sparse_mla_decode_paged_launcher': (None, [_P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int,
                                                 c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
                                                 _P]),
+    'sparse_mla_decode_fp8_paged_launcher': (None, [_P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int,
+                                                    c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
+                                                    _P]),
     'sparse_mla_decode_num_splits': (c_int, [c_int, c_int, c_int, c_int]),
     'sparse_mla_decode_workspace_bytes': (c_size_t, [c_int, c_int, c_int, c_int]),
     'mla_latent_quant_launcher': (None, [_P, _P, c_long, c_int, _P]),
@@ -337,6 +340,37 @@ def sparse_mla_decode_fp8_launch(out, q, kv_fp8, idx, workspace, sm_scale=192 **
         _ptr(out), _ptr(q), _ptr(kv_fp8), _ptr(idx), _ptr(workspace), workspace.numel(), B, H, N, topk, d_qk, d_v,
         float(sm_scale), 0 if out.dtype == torch.bfloat16 else 1, config, _stream(stream))
     check_status('sparse_mla_decode_fp8_launcher')
+    return out
+
+
+def sparse_mla_decode_fp8_paged_launch(out, q, kv_pool_fp8, block_table, idx, workspace, sm_scale=192 ** -0.5,
+                                       config=0, stream=None):
+    """As ``sparse_mla_decode_paged_launch`` over kv_pool_fp8 [n_pages, page_size, 656] uint8 (the e4m3 storage
+    form); ``workspace``: at least ``sparse_mla_fp8_workspace_bytes`` bytes."""
+    import torch
+    _device_contiguous(out=out, q=q, kv_pool_fp8=kv_pool_fp8, idx=idx, workspace=workspace)
+    B, H, d_qk = q.shape
+    n_pages, page_size = kv_pool_fp8.shape[0], kv_pool_fp8.shape[1]
+    topk = idx.shape[1]
+    d_v = out.shape[2]
+    _require(q.dtype == torch.bfloat16 and kv_pool_fp8.dtype == torch.uint8, 'sparse_mla_fp8: q bf16, kv_pool_fp8 uint8')
+    _require(out.dtype in (torch.bfloat16, torch.float32), 'sparse_mla_fp8: out must be bf16 or fp32')
+    _require(idx.dtype == torch.int32, 'sparse_mla_fp8: idx must be int32')
+    _require(tuple(kv_pool_fp8.shape) == (n_pages, page_size, LATENT_ROW_BYTES) and tuple(idx.shape) == (B, topk),
+             'sparse_mla_fp8: kv_pool_fp8 [n_pages, page, 656], idx [B, topk]')
+    _require(tuple(out.shape) == (B, H, d_v), 'sparse_mla_fp8: out shape')
+    max_pages = 0
+    if block_table is not None:
+        _device_contiguous(block_table=block_table)
+        _require(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.shape[0] == B,
+                 'sparse_mla_fp8: block_table must be int32 [B, max_pages]')
+        max_pages = block_table.shape[1]
+    library().sparse_mla_decode_fp8_paged_launcher(
+        _ptr(out), _ptr(q), _ptr(kv_pool_fp8), _ptr(block_table) if block_table is not None else None,
+        _ptr(idx), _ptr(workspace), workspace.numel() * workspace.element_size(), B, H, n_pages,
+        page_size, max_pages, topk, d_qk, d_v, float(sm_scale),
+        0 if out.dtype == torch.bfloat16 else 1, config, _stream(stream))
+    check_status('sparse_mla_decode_fp8_paged_launcher')
     return out
 
 

@@ -22,6 +22,7 @@
 #include <stdint.h>
 
 #include "launch_status.hpp"
+#include "mla_addressing.hpp"
 #include "moe_common.hpp"
 
 extern "C" size_t sparse_mla_decode_workspace_bytes(int batch, int n_heads, int topk, int config);
@@ -104,17 +105,17 @@ __global__ __launch_bounds__(256) void mla_latent_gather_kernel(const uint8_t* _
                                                                 const int* __restrict__ idx,
                                                                 __hip_bfloat16* __restrict__ rows_out,
                                                                 int* __restrict__ idx_out, int n_kv_rows,
-                                                                int topk) {
+                                                                int topk, mla::KvAddressing kva) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int b = blockIdx.y;
     const int first = blockIdx.x * ROWS_PER_WG + wave * ROWS_PER_WAVE;
     if (first >= topk) return;  // (no barrier in this kernel)
-    const uint8_t* cache_b = cache + (size_t)b * n_kv_rows * ROW_FP8_BYTES;
-    // keys of this wavefront's rows, one per lane, then broadcast
+    const uint8_t* cache_b = cache + (size_t)b * kva.batch_rows * ROW_FP8_BYTES;
+    // rows of this wavefront's entries (block table, bounds), one per lane, then broadcast
     int my_key = -1;
-    if (lane < ROWS_PER_WAVE && first + lane < topk) my_key = idx[(size_t)b * topk + first + lane];
-    if (my_key < 0 || my_key >= n_kv_rows) my_key = -1;
+    if (lane < ROWS_PER_WAVE && first + lane < topk)
+        my_key = mla::resolve_key(idx[(size_t)b * topk + first + lane], b, kva, n_kv_rows);
     if (lane < ROWS_PER_WAVE && first + lane < topk) idx_out[(size_t)b * topk + first + lane] = my_key < 0 ? -1 : first + lane;
 
     uintx4 chunk[ROWS_PER_WAVE];
@@ -189,14 +190,12 @@ extern "C" size_t sparse_mla_decode_fp8_workspace_bytes(int batch, int n_heads, 
            align16((size_t)batch * topk * ROW_BF16_BYTES) + align16((size_t)batch * topk * sizeof(int));
 }
 
-// sparse_mla_decode_launcher over a cache in the 656-byte form: kv_fp8 [batch, n_kv_rows, 656] bytes,
-// 16-byte aligned; everything else as there (idx entries < 0 or >= n_kv_rows are padding). The result
-// equals sparse_mla_decode_launcher on the dequantised cache bit for bit.
-extern "C" void sparse_mla_decode_fp8_launcher(void* out, const void* q, const void* kv_fp8,
-                                               const int* idx, void* workspace, size_t workspace_bytes,
-                                               int batch, int n_heads, int n_kv_rows, int topk, int d_qk,
-                                               int d_v, float sm_scale, int out_dtype, int config,
-                                               hipStream_t stream) {
+namespace {
+
+void launch_decode_fp8(void* out, const void* q, const void* kv_fp8, const int* idx, void* workspace,
+                       size_t workspace_bytes, int batch, int n_heads, int n_kv_rows, int topk, int d_qk,
+                       int d_v, float sm_scale, int out_dtype, int config, const mla::KvAddressing& kva,
+                       hipStream_t stream) {
     if (batch <= 0 || n_heads <= 0 || topk <= 0) return;
     if (d_qk != ROW_VALUES || d_v != LATENT || n_kv_rows <= 0 || batch > 65535) {
         caa::set_status(CAA_UNSUPPORTED_SHAPE);
@@ -217,7 +216,46 @@ extern "C" void sparse_mla_decode_fp8_launcher(void* out, const void* q, const v
     int* compact_idx = reinterpret_cast<int*>(ws + base_bytes + align16((size_t)batch * topk * ROW_BF16_BYTES));
     const dim3 grid((topk + ROWS_PER_WG - 1) / ROWS_PER_WG, batch);
     mla_latent_gather_kernel<<<grid, 256, 0, stream>>>(static_cast<const uint8_t*>(kv_fp8), idx, rows,
-                                                       compact_idx, n_kv_rows, topk);
+                                                       compact_idx, n_kv_rows, topk, kva);
     sparse_mla_decode_launcher(out, q, rows, compact_idx, workspace, base_bytes, batch, n_heads, topk, topk,
                                d_qk, d_v, sm_scale, out_dtype, config, stream);
+}
+
+}  // namespace
+
+// sparse_mla_decode_launcher over a cache in the 656-byte form: kv_fp8 [batch, n_kv_rows, 656] bytes,
+// 16-byte aligned; everything else as there (idx entries < 0 or >= n_kv_rows are padding). The result
+// equals sparse_mla_decode_launcher on the dequantised cache bit for bit.
+extern "C" void sparse_mla_decode_fp8_launcher(void* out, const void* q, const void* kv_fp8,
+                                               const int* idx, void* workspace, size_t workspace_bytes,
+                                               int batch, int n_heads, int n_kv_rows, int topk, int d_qk,
+                                               int d_v, float sm_scale, int out_dtype, int config,
+                                               hipStream_t stream) {
+    const mla::KvAddressing kva{nullptr, 0, 0, n_kv_rows};
+    launch_decode_fp8(out, q, kv_fp8, idx, workspace, workspace_bytes, batch, n_heads, n_kv_rows, topk, d_qk,
+                      d_v, sm_scale, out_dtype, config, kva, stream);
+}
+
+// The same over a paged cache in the 656-byte form: kv_pool_fp8 [n_pages, page_size, 656] bytes shared by
+// all requests; block_table, idx and limits as sparse_mla_decode_paged_launcher (with a block table idx holds
+// logical positions, without one rows of the pool). The workspace is that of sparse_mla_decode_fp8_launcher.
+extern "C" void sparse_mla_decode_fp8_paged_launcher(void* out, const void* q, const void* kv_pool_fp8,
+                                                     const int* block_table, const int* idx,
+                                                     void* workspace, size_t workspace_bytes, int batch,
+                                                     int n_heads, int n_pages, int page_size,
+                                                     int max_pages_per_request, int topk, int d_qk, int d_v,
+                                                     float sm_scale, int out_dtype, int config,
+                                                     hipStream_t stream) {
+    if (batch <= 0 || n_heads <= 0 || topk <= 0) return;
+    if (n_pages <= 0 || page_size <= 0 || (page_size & (page_size - 1)) != 0 ||
+        (long long)n_pages * page_size > 0x7fffffffll ||
+        (block_table != nullptr && max_pages_per_request <= 0)) {
+        caa::set_status(CAA_UNSUPPORTED_SHAPE);
+        return;
+    }
+    int page_shift = 0;
+    while ((1 << page_shift) < page_size) ++page_shift;
+    const mla::KvAddressing kva{block_table, max_pages_per_request, page_shift, 0};
+    launch_decode_fp8(out, q, kv_pool_fp8, idx, workspace, workspace_bytes, batch, n_heads,
+                      n_pages * page_size, topk, d_qk, d_v, sm_scale, out_dtype, config, kva, stream);
 }

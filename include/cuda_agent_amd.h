@@ -186,6 +186,16 @@ void sparse_mla_decode_fp8_launcher(void* out, const void* q, const void* kv_fp8
                                     int n_kv_rows, int topk, int d_qk, int d_v, float sm_scale,
                                     int out_dtype, int config, hipStream_t stream);
 
+/* sparse_mla_decode_fp8_launcher over a paged cache: kv_pool_fp8 [n_pages, page_size, 656] bytes shared by all
+ * requests; block_table, idx, page limits as sparse_mla_decode_paged_launcher; workspace as
+ * sparse_mla_decode_fp8_launcher. */
+void sparse_mla_decode_fp8_paged_launcher(void* out, const void* q, const void* kv_pool_fp8,
+                                          const int* block_table, const int* idx, void* workspace,
+                                          size_t workspace_bytes, int batch, int n_heads, int n_pages,
+                                          int page_size, int max_pages_per_request, int topk, int d_qk,
+                                          int d_v, float sm_scale, int out_dtype, int config,
+                                          hipStream_t stream);
+
 /* Index scores of the sparse-attention indexer, decode step (caller-side neighbour of the top-k
  * selection below; same launcher pattern agent_workdir/kernels/axpby.cu:12-20):
  *   scores[b, t] = sum_h w[b, h] * max(0, scale * q[b, h, :] . k_cache[b, t, :])  for t < lengths[b]

@@ -110,3 +110,38 @@ def test_rejects_bad_arguments(capi, dev):
         capi.sparse_mla_decode_fp8_launch(out, q, cache, idx,
                                           torch.empty(capi.sparse_mla_workspace_bytes(1, 128, 32), dtype=torch.uint8, device=dev))
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize('page', [16, 64])
+def test_paged_fp8_cache(capi, dev, page):
+    # the pages of a contiguous e4m3 cache scattered into a pool: the same result bit for bit, with a block table
+    # (logical positions) and without one (pool rows); an unmapped page is padding
+    gen = torch.Generator().manual_seed(60 + page)
+    B, H, N, topk = 3, 128, 1024, 256
+    q, kv, idx = mla.mla_make_inputs(B, H, N, topk, generator=gen)
+    cache = make_cache(capi, dev, kv)
+    per_req = N // page
+    n_pages = B * per_req + 3
+    order = torch.randperm(n_pages, generator=gen)[:B * per_req]
+    pool = torch.randint(0, 255, (n_pages, page, 656), generator=gen).to(torch.uint8)
+    pool[order] = cache.cpu().reshape(B * per_req, page, 656)
+    table = order.reshape(B, per_req).int()
+    want = run_fp8(capi, dev, q, cache, idx, torch.float32)
+
+    def run_paged(table_arg, idx_arg):
+        out = torch.full((B, H, 512), float('nan'), device=dev)
+        ws = torch.empty(capi.sparse_mla_fp8_workspace_bytes(B, H, topk), dtype=torch.uint8, device=dev)
+        capi.sparse_mla_decode_fp8_paged_launch(out, q.to(dev), pool.to(dev), None if table_arg is None else table_arg.to(dev),
+                                                idx_arg.to(dev), ws)
+        torch.cuda.synchronize()
+        return out.cpu()
+
+    assert torch.equal(run_paged(table, idx), want)
+    rows = mla.resolve_paged_indices(idx, table, page, n_pages * page).int()
+    assert torch.equal(run_paged(None, rows), want)
+    # one page of request 1 unmapped: its positions become padding
+    table2 = table.clone()
+    table2[1, 2] = -1
+    idx_masked = idx.clone()
+    idx_masked[1][(idx[1] >= 2 * page) & (idx[1] < 3 * page)] = -1
+    assert torch.equal(run_paged(table2, idx), run_fp8(capi, dev, q, cache, idx_masked, torch.float32))
