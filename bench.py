@@ -264,6 +264,15 @@ def bench_router(torch, capi, dev, steps, warmup, cpu_baseline, prefill):
         capi.moe_route_grouped_launch(ids, wts, logits, bias, 8, 4, True, 2.5)
 
     sec = timed_launches(torch, launch, steps, warmup)
+    # the same chain with the weight prepared once as three bf16 planes (projection on the bf16 matrix cores)
+    planes = torch.empty(3, E, H, dtype=torch.bfloat16, device=dev)
+    capi.moe_router_split_weight_launch(planes, w)
+
+    def launch_split(i):
+        capi.moe_router_logits_split_launch(logits, x, planes, ws)
+        capi.moe_route_grouped_launch(ids, wts, logits, bias, 8, 4, True, 2.5)
+
+    sec_split = timed_launches(torch, launch_split, steps, warmup)
     flops = 2 * T * H * E
     nbytes_alg = E * H * 4 + T * H * 2 + T * E * 4 + 2 * T * k * 4
     if prefill:
@@ -284,6 +293,8 @@ def bench_router(torch, capi, dev, steps, warmup, cpu_baseline, prefill):
             roofline=dict(bound="hbm", achieved=nbytes_alg / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
                           frac=nbytes_alg / sec / 1e9 / HBM_PEAK_GBS, traffic=None),
             algorithmic_bytes=nbytes_alg)
+    res['with_split_weight'] = dict(ms_per_step=sec_split * 1e3, kernel="moe_router_gemm_split_kernel",
+                                    note="fp32 weight as three bf16 planes, 3 exact bf16 products per weight")
     if cpu_baseline:
         cores = len(os.sched_getaffinity(0))
         torch.set_num_threads(cores)

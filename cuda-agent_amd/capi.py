@@ -51,6 +51,8 @@ SIGNATURES = {
     'moe_router_logits_num_splits': (c_int, [c_int, c_int, c_int]),
     'moe_router_logits_workspace_bytes': (c_size_t, [c_int, c_int, c_int]),
     'moe_router_logits_launcher': (None, [_P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int, c_int, _P]),
+    'moe_router_split_weight_launcher': (None, [_P, _P, c_int, c_int, _P]),
+    'moe_router_logits_split_launcher': (None, [_P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int, _P]),
     'moe_route_grouped_launcher': (None, [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
                                           c_int, _P]),
     'moe_sort_launcher': (None, [_P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P]),
@@ -559,6 +561,37 @@ def moe_router_logits_launch(logits, x, w, workspace=None, stream=None):
     library().moe_router_logits_launcher(_ptr(logits), _ptr(x), _ptr(w), ws_ptr, ws_bytes, T, H, E,
                                          0 if x.dtype == torch.float32 else 1, 0, _stream(stream))
     check_status('moe_router_logits_launcher')
+    return logits
+
+
+def moe_router_split_weight_launch(planes, w, stream=None):
+    """planes [3, E, H] bf16 <- the three bf16 numbers whose sum is w [E, H] fp32 (done once per weight)."""
+    import torch
+    _device_contiguous(planes=planes, w=w)
+    E, H = w.shape
+    _require(w.dtype == torch.float32 and planes.dtype == torch.bfloat16 and tuple(planes.shape) == (3, E, H),
+             'moe_router_split_weight: w fp32 [E, H], planes bf16 [3, E, H]')
+    library().moe_router_split_weight_launcher(_ptr(planes), _ptr(w), E, H, _stream(stream))
+    check_status('moe_router_split_weight_launcher')
+    return planes
+
+
+def moe_router_logits_split_launch(logits, x, planes, workspace=None, stream=None):
+    """``moe_router_logits_launch`` for a bf16 x and the weight given as its three bf16 planes [3, E, H]."""
+    import torch
+    _device_contiguous(logits=logits, x=x, planes=planes)
+    T, H = x.shape
+    E = planes.shape[1]
+    _require(x.dtype == planes.dtype == torch.bfloat16 and logits.dtype == torch.float32,
+             'moe_router_logits_split: x and planes bf16, logits fp32')
+    _require(tuple(planes.shape) == (3, E, H) and tuple(logits.shape) == (T, E), 'moe_router_logits_split: shapes')
+    ws_ptr, ws_bytes = c_void_p(None), 0
+    if workspace is not None:
+        _device_contiguous(workspace=workspace)
+        ws_ptr, ws_bytes = _ptr(workspace), workspace.numel() * workspace.element_size()
+    library().moe_router_logits_split_launcher(_ptr(logits), _ptr(x), _ptr(planes), ws_ptr, ws_bytes, T, H, E, 0,
+                                               _stream(stream))
+    check_status('moe_router_logits_split_launcher')
     return logits
 
 

@@ -17,6 +17,14 @@
 // Few tokens: K is cut into n_splits ranges (grid z) so that the weight matrix is streamed by
 // many CUs; partial sums go to a caller-provided scratch and a second kernel adds them in
 // ascending split order, so the result does not depend on timing.
+//
+// Split-weight form (moe_router_split_weight_launcher + moe_router_logits_split_launcher): an fp32
+// weight is the exact sum of three bf16 numbers (its 24 significand bits cut into 8 + 8 + 8), and a
+// product of two bf16 numbers is exact in fp32. With the weight stored once as those three planes the
+// projection of a bf16 x runs on the bf16 matrix cores (v_mfma_f32_32x32x16_bf16: 8 times the rate of
+// the fp32 shape, three products per weight) and still differs from an fp32 reference by the order of the
+// additions only. At that rate the operand loads are what matters: rows are fetched as whole lines and
+// turned into the operand layout through a small LDS buffer private to the wavefront.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -27,6 +35,7 @@ namespace {
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int K_CHUNK = 64;
 
@@ -98,6 +107,104 @@ __global__ __launch_bounds__(256) void moe_router_gemm_kernel(const X* __restric
         for (int s = 0; s < 32; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[s], b1[s], acc, 0, 0, 0);
     }
     // result register i of a lane: token 8*(i/4) + 4*half + i%4 of the tile, expert `row`
+    float* dst = out + (size_t)blockIdx.z * tokens * n_experts;
+    if (e0 + row < n_experts) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int tt = t0 + 8 * (i / 4) + 4 * half + (i % 4);
+            if (tt < tokens) dst[(size_t)tt * n_experts + e0 + row] = acc[i];
+        }
+    }
+}
+
+// ---- split-weight form ---------------------------------------------------------------------------------
+
+// w [n] fp32 -> planes [3][n] bf16 with hi + mid + lo == w exactly: hi = the upper 16 bits of w, mid the upper
+// 16 bits of w - hi, lo = w - hi - mid (at most 8 significant bits are left, so it is a bf16 number)
+__global__ __launch_bounds__(256) void moe_router_split_kernel(const float* __restrict__ w,
+                                                               uint16_t* __restrict__ planes, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const float v = w[i];
+    const uint32_t hi = __float_as_uint(v) & 0xffff0000u;
+    const float r1 = v - __uint_as_float(hi);
+    const uint32_t mid = __float_as_uint(r1) & 0xffff0000u;
+    const float r2 = r1 - __uint_as_float(mid);
+    planes[i] = (uint16_t)(hi >> 16);
+    planes[n + i] = (uint16_t)(mid >> 16);
+    planes[2 * n + i] = (uint16_t)(__float_as_uint(r2) >> 16);
+}
+
+// grid as moe_router_gemm_kernel. A wavefront owns 32 tokens x 32 experts; per 64 values of k it fetches
+// four tiles of 32 rows x 128 bytes (x and the three weight planes), each with 4 load instructions of whole
+// lines (lane l: 16-byte chunk l % 8 of row 8*j + l / 8), and passes them one after the other through its
+// 4 KB LDS buffer (chunk c of row r at slot c ^ ((r >> 1) & 7)) into the operand layout: lane (row, half)
+// holds values [32*half, +32) of its row, 8 per MFMA step. No barrier: the buffer is private and the LDS
+// operations of a wavefront execute in order.
+__global__ __launch_bounds__(256) void moe_router_gemm_split_kernel(const uint16_t* __restrict__ x,
+                                                                    const uint16_t* __restrict__ planes,
+                                                                    float* __restrict__ out, int tokens,
+                                                                    int hidden, int n_experts,
+                                                                    int chunks_per_split) {
+    __shared__ u32x4 s_tile[4][32 * 8];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int row = lane & 31;
+    const int half = lane >> 5;
+    const int t0 = blockIdx.x * 64 + (wave & 1) * 32;
+    const int e0 = blockIdx.y * 64 + (wave >> 1) * 32;
+    if (t0 >= tokens || e0 >= n_experts) return;  // (no barrier in this kernel)
+    u32x4* tile = s_tile[wave];
+    const int chunk_begin = blockIdx.z * chunks_per_split;
+    int chunk_end = chunk_begin + chunks_per_split;
+    const int n_chunks = hidden / K_CHUNK;
+    if (chunk_end > n_chunks) chunk_end = n_chunks;
+    const size_t plane = (size_t)n_experts * hidden;
+
+    // fill side: rows 8*j + lane/8 of the tile, chunk lane%8 (rows beyond the end repeat the last valid one)
+    const u32x4* src[4][4];  // [x, hi, mid, lo][instruction]
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int r = 8 * j + (lane >> 3);
+        const int t = t0 + r < tokens ? t0 + r : tokens - 1;
+        const int e = e0 + r < n_experts ? e0 + r : n_experts - 1;
+        src[0][j] = reinterpret_cast<const u32x4*>(x + (size_t)t * hidden) + (lane & 7);
+#pragma unroll
+        for (int p = 0; p < 3; ++p)
+            src[1 + p][j] = reinterpret_cast<const u32x4*>(planes + p * plane + (size_t)e * hidden) + (lane & 7);
+    }
+    u32x4 raw[4][4];
+    auto load_chunk = [&](int c) {
+#pragma unroll
+        for (int m = 0; m < 4; ++m)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) raw[m][j] = src[m][j][(size_t)c * (K_CHUNK * 2 / 16)];
+    };
+    // operand of matrix m: through the buffer
+    bf16x8 op[4][4];
+    auto stage = [&](int m) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int r = 8 * j + (lane >> 3);
+            tile[r * 8 + ((lane & 7) ^ ((r >> 1) & 7))] = raw[m][j];
+        }
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+            op[m][s] = __builtin_bit_cast(bf16x8, tile[row * 8 + ((4 * half + s) ^ ((row >> 1) & 7))]);
+    };
+
+    floatx16 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (chunk_begin < chunk_end) load_chunk(chunk_begin);
+    for (int c = chunk_begin; c < chunk_end; ++c) {
+#pragma unroll
+        for (int m = 0; m < 4; ++m) stage(m);
+        if (c + 1 < chunk_end) load_chunk(c + 1);  // in flight under the MFMAs below
+        // smallest terms first
+#pragma unroll
+        for (int p = 3; p >= 1; --p)
+#pragma unroll
+            for (int s = 0; s < 4; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(op[0][s], op[p][s], acc, 0, 0, 0);
+    }
     float* dst = out + (size_t)blockIdx.z * tokens * n_experts;
     if (e0 + row < n_experts) {
 #pragma unroll
@@ -187,6 +294,58 @@ extern "C" void moe_router_logits_launcher(float* logits, const void* x, const f
         moe_router_gemm_kernel<uint16_t><<<grid, 256, 0, stream>>>(
             static_cast<const uint16_t*>(x), w, out, tokens, hidden, n_experts, chunks_per_split);
     }
+    if (splits > 1) {
+        const size_t count = (size_t)tokens * n_experts;
+        moe_router_reduce_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>(
+            static_cast<const float*>(workspace), logits, count, splits);
+    }
+}
+
+// planes [3, n_experts, hidden] bf16 (written) from w [n_experts, hidden] fp32: the three bf16 numbers whose
+// sum is the weight, for moe_router_logits_split_launcher. Done once per weight.
+extern "C" void moe_router_split_weight_launcher(void* planes, const float* w, int n_experts, int hidden,
+                                                 hipStream_t stream) {
+    if (n_experts <= 0 || hidden <= 0) return;
+    if (!planes || !w) {
+        caa::set_status(CAA_BAD_ARGUMENT);
+        return;
+    }
+    const size_t n = (size_t)n_experts * hidden;
+    moe_router_split_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(w, static_cast<uint16_t*>(planes), n);
+}
+
+// moe_router_logits_launcher for a bf16 x and a weight given as the planes above: the same logits up to the
+// order of the fp32 additions, on the bf16 matrix cores. Sizes, scratch (moe_router_logits_workspace_bytes)
+// and limits as there; x and planes 16-byte aligned, hidden a multiple of 64.
+extern "C" void moe_router_logits_split_launcher(float* logits, const void* x, const void* planes,
+                                                 void* workspace, size_t workspace_bytes, int tokens,
+                                                 int hidden, int n_experts, int config, hipStream_t stream) {
+    (void)config;
+    if (tokens <= 0 || n_experts <= 0) return;
+    if (hidden <= 0 || hidden % K_CHUNK != 0 || (tokens + 63) / 64 > 0x7fffffff / 64 ||
+        (n_experts + 63) / 64 > 65535) {
+        caa::set_status(CAA_UNSUPPORTED_SHAPE);
+        return;
+    }
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(planes) |
+                           reinterpret_cast<uintptr_t>(workspace);
+    if (!logits || !x || !planes || (bits & 15u) != 0) {
+        caa::set_status(CAA_BAD_ARGUMENT);
+        return;
+    }
+    const int splits = pick_router_splits(tokens, hidden, n_experts);
+    const size_t need = splits <= 1 ? 0 : (size_t)splits * tokens * n_experts * sizeof(float);
+    if (need > 0 && (!workspace || workspace_bytes < need)) {
+        caa::set_status(CAA_WORKSPACE_TOO_SMALL);
+        return;
+    }
+    const int n_chunks = hidden / K_CHUNK;
+    const int chunks_per_split = (n_chunks + splits - 1) / splits;
+    float* out = splits > 1 ? static_cast<float*>(workspace) : logits;
+    const dim3 grid((tokens + 63) / 64, (n_experts + 63) / 64, splits);
+    moe_router_gemm_split_kernel<<<grid, 256, 0, stream>>>(static_cast<const uint16_t*>(x),
+                                                           static_cast<const uint16_t*>(planes), out, tokens,
+                                                           hidden, n_experts, chunks_per_split);
     if (splits > 1) {
         const size_t count = (size_t)tokens * n_experts;
         moe_router_reduce_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>(

@@ -282,6 +282,19 @@ void moe_router_logits_launcher(float* logits, const void* x, const float* w, vo
                                 size_t workspace_bytes, int tokens, int hidden, int n_experts,
                                 int x_dtype, int config, hipStream_t stream);
 
+/* The router weight as three bf16 planes [3, n_experts, hidden] whose sum is w exactly (the 24 significand
+ * bits of an fp32 number cut 8 + 8 + 8); prepared once per weight for the launcher below. */
+void moe_router_split_weight_launcher(void* planes, const float* w, int n_experts, int hidden,
+                                      hipStream_t stream);
+
+/* moe_router_logits_launcher for a bf16 x and the weight given as those planes: every product is exact in
+ * fp32, so the logits differ from the fp32 launcher's by the order of the additions only, and the
+ * projection runs on the bf16 matrix cores. Scratch (moe_router_logits_workspace_bytes), sizes and limits as
+ * moe_router_logits_launcher; x and planes 16-byte aligned. */
+void moe_router_logits_split_launcher(float* logits, const void* x, const void* planes, void* workspace,
+                                      size_t workspace_bytes, int tokens, int hidden, int n_experts,
+                                      int config, hipStream_t stream);
+
 /* Group-limited routing with a selection bias, the router of DeepSeek-V3-style layers (caller-
  * side neighbour of moe_route_launcher; same launcher pattern):
  *   score = sigmoid(logit), choice = score + bias; a group (n_experts/n_group consecutive

@@ -162,6 +162,17 @@ def router_logits(x, w):
     return x.float() @ w.float().T
 
 
+def split_bf16x3(w):
+    """w fp32 -> planes [3, ...] bf16 with planes.float().sum(0) == w exactly: hi = w with the lower 16 bits cleared,
+    mid = (w - hi) with the lower 16 bits cleared, lo = w - hi - mid (8 significant bits are left: a bf16 number)."""
+    bits = w.contiguous().view(torch.int32)
+    hi = (bits & -65536).view(torch.float32)
+    r1 = w - hi
+    mid = (r1.contiguous().view(torch.int32) & -65536).view(torch.float32)
+    lo = r1 - mid
+    return torch.stack([hi, mid, lo]).bfloat16()
+
+
 def route_grouped(logits, bias, top_k, n_group, topk_group, normalise=True, routed_scaling_factor=1.0):
     """Group-limited routing with a selection bias.
 

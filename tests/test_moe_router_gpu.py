@@ -177,6 +177,60 @@ def test_projection_then_grouped_routing_at_prefill_size(capi, dev):
     assert differing <= 8, differing        # logits differ in the last place: 1 token in 1000 may flip
 
 
+# ---- router projection with the weight split into three bf16 planes -------------------------------------------
+
+def run_logits_split(capi, dev, x, w):
+    T, H = x.shape
+    E = w.shape[0]
+    planes = torch.empty(3, E, H, dtype=torch.bfloat16, device=dev)
+    capi.moe_router_split_weight_launch(planes, w.to(dev))
+    logits = torch.full((T, E), float('nan'), device=dev)
+    nbytes = capi.moe_router_logits_workspace_bytes(T, H, E)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev) if nbytes else None
+    capi.moe_router_logits_split_launch(logits, x.to(dev), planes, ws)
+    torch.cuda.synchronize()
+    return logits.cpu(), planes.cpu()
+
+
+@pytest.mark.parametrize('shape', [(64, 7168, 256), (1, 64, 32), (100, 448, 72), (700, 1024, 256), (33, 128, 1),
+                                   (130, 2048, 384)])
+def test_split_weight_logits_match_float64(capi, dev, shape):
+    T, H, E = shape
+    gen = torch.Generator().manual_seed(T + E + 1)
+    x = torch.randn(T, H, generator=gen).bfloat16()
+    w = torch.randn(E, H, generator=gen) * H ** -0.5
+    w[0, :4] = torch.tensor([0.0, 1e-30, -3e38, 2.0 ** -120])
+    got, planes = run_logits_split(capi, dev, x, w)
+    # the planes are the oracle's, and their sum is the weight, bit for bit
+    assert torch.equal(planes.view(torch.int16), moe.split_bf16x3(w).view(torch.int16))
+    assert torch.equal((planes[0].float() + planes[1].float()) + planes[2].float(), w)
+    w[0, 2] = 0.0                                  # (keep the reference finite)
+    got, _ = run_logits_split(capi, dev, x, w)
+    want = x.double() @ w.double().T
+    assert torch.isfinite(got).all()
+    assert ((got.double() - want).abs() <= logits_bound(x, w)).all()
+    err = (got.double() - want).abs().max().item()
+    ref_err = (moe.router_logits(x, w).double() - want).abs().max().item()
+    assert err <= 4 * ref_err + 1e-7
+
+
+def test_split_weight_logits_exact_on_integers_and_routing_chain(capi, dev):
+    gen = torch.Generator().manual_seed(53)
+    x = torch.randint(-8, 9, (96, 512), generator=gen).float().bfloat16()
+    w = torch.randint(-8, 9, (64, 512), generator=gen).float()
+    got, _ = run_logits_split(capi, dev, x, w)
+    assert torch.equal(got, x.float() @ w.T)
+    # hidden states -> logits -> experts at prefill size, against the oracle's chain
+    T, H, E = 8192, 1024, 256
+    x = torch.randn(T, H, generator=gen).bfloat16()
+    w = torch.randn(E, H, generator=gen) * H ** -0.5
+    bias = 0.1 * torch.randn(E, generator=gen)
+    logits, _ = run_logits_split(capi, dev, x, w)
+    ids, _ = run_kernel(capi, dev, logits, bias, 8, 8, 4, True, 2.5)
+    want_ids, _, _ = moe.route_grouped(moe.router_logits(x, w), bias, 8, 8, 4, True, 2.5)
+    assert (ids != want_ids).any(dim=1).sum().item() <= 8
+
+
 def test_router_logits_rejects_bad_arguments(capi, dev):
     logits = torch.zeros(4, 32, device=dev)
     w = torch.zeros(32, 96, device=dev)

@@ -369,3 +369,22 @@ def test_rmsnorm_bf16_closed_form_and_golden():
     # the module uses rsqrt, this restatement 1/sqrt: an fp32 ulp of the factor can move a value across a bf16 boundary
     assert (got.float() == want).float().mean() >= 0.995
     assert ((got.float() - want).abs() <= want.abs() * 2.0 ** -7).all()
+
+
+def test_split_bf16x3_is_exact():
+    gen = torch.Generator().manual_seed(77)
+    w = torch.randn(50, 64, generator=gen) * torch.exp(4 * torch.randn(50, 1, generator=gen))
+    w[0, :5] = torch.tensor([0.0, -0.0, 1e-30, 3e38, 2.0 ** -120])
+    planes = moe.split_bf16x3(w)
+    assert planes.dtype == torch.bfloat16 and planes.shape == (3, 50, 64)
+    assert torch.equal((planes[0].float() + planes[1].float()) + planes[2].float(), w)
+    assert torch.equal(planes.double().sum(0), w.double())
+    # the first plane is w with its lower 16 bits cleared; the planes shrink by 2^-8 each
+    assert torch.equal(planes[0].float().view(torch.int32), w.view(torch.int32) & -65536)
+    assert (planes[1].float().abs() <= planes[0].float().abs() * 2.0 ** -7 + 1e-45).all()
+    assert (planes[2].float().abs() <= planes[0].float().abs() * 2.0 ** -15 + 1e-45).all()
+    # so a bf16 x times the planes gives the fp32 product terms exactly
+    x = torch.randn(64, generator=gen).bfloat16()
+    exact = (x.double()[None, :] * w.double()).sum(dim=1)
+    via_planes = sum((x.double()[None, :] * planes[i].double()).sum(dim=1) for i in range(3))
+    torch.testing.assert_close(via_planes, exact, rtol=1e-14, atol=0)
