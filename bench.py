@@ -293,7 +293,8 @@ def bench_router(torch, capi, dev, steps, warmup, cpu_baseline, prefill):
             roofline=dict(bound="hbm", achieved=nbytes_alg / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
                           frac=nbytes_alg / sec / 1e9 / HBM_PEAK_GBS, traffic=None),
             algorithmic_bytes=nbytes_alg)
-    res['with_split_weight'] = dict(ms_per_step=sec_split * 1e3, kernel="moe_router_gemm_split_kernel",
+    res['with_split_weight'] = dict(ms_per_step=sec_split * 1e3,
+                                    kernel="moe_router_gemm_split_tiled_kernel" if prefill else "moe_router_gemm_split_kernel",
                                     note="fp32 weight as three bf16 planes, 3 exact bf16 products per weight")
     if cpu_baseline:
         cores = len(os.sched_getaffinity(0))

@@ -215,6 +215,107 @@ __global__ __launch_bounds__(256) void moe_router_gemm_split_kernel(const uint16
     }
 }
 
+// The same product for many tokens: a workgroup owns 128 tokens x 64 experts and shares its operand tiles
+// through LDS (per 64 values of k: 128 rows of x and 3 x 64 rows of planes, 128 bytes each = 40 KB, two
+// stages). Every lane fetches 10 chunks of 16 bytes per stage (whole lines: 8 lanes per row), stores them
+// swizzled as above, and after ONE barrier per stage each wavefront (64 tokens x 32 experts) reads its two x
+// tiles and three plane tiles in operand layout. The per-wavefront kernel above asks its CU's L1 for 170
+// bytes per clock at the bf16 MFMA rate; this one for 52.
+constexpr int BIG_TOKENS = 128;
+constexpr int BIG_EXPERTS = 64;
+constexpr int BIG_STAGE = (BIG_TOKENS + 3 * BIG_EXPERTS) * 8;  // 16-byte slots per stage (40 KB)
+
+__global__ __launch_bounds__(256) void moe_router_gemm_split_tiled_kernel(const uint16_t* __restrict__ x,
+                                                                          const uint16_t* __restrict__ planes,
+                                                                          float* __restrict__ out, int tokens,
+                                                                          int hidden, int n_experts) {
+    __shared__ u32x4 s_stage[2][BIG_STAGE];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int row = lane & 31;
+    const int half = lane >> 5;
+    const int t0 = blockIdx.x * BIG_TOKENS;
+    const int e0 = blockIdx.y * BIG_EXPERTS;
+    const int n_chunks = hidden / K_CHUNK;
+    const size_t plane = (size_t)n_experts * hidden;
+
+    // fill side: slot tid + 256*i of the stage, i < 10; rows 0..127 are x, then 64 rows of each plane
+    const u32x4* src[10];
+    int dst[10];
+#pragma unroll
+    for (int i = 0; i < 10; ++i) {
+        const int r = (tid + 256 * i) >> 3;  // row of the stage
+        const int c = tid & 7;
+        if (r < BIG_TOKENS) {
+            const int t = t0 + r < tokens ? t0 + r : tokens - 1;
+            src[i] = reinterpret_cast<const u32x4*>(x + (size_t)t * hidden) + c;
+        } else {
+            const int p = (r - BIG_TOKENS) / BIG_EXPERTS;
+            const int er = (r - BIG_TOKENS) % BIG_EXPERTS;
+            const int e = e0 + er < n_experts ? e0 + er : n_experts - 1;
+            src[i] = reinterpret_cast<const u32x4*>(planes + p * plane + (size_t)e * hidden) + c;
+        }
+        dst[i] = r * 8 + (c ^ ((r >> 1) & 7));
+    }
+    u32x4 raw[10];
+    auto load_chunk = [&](int c) {
+#pragma unroll
+        for (int i = 0; i < 10; ++i) raw[i] = src[i][(size_t)c * (K_CHUNK * 2 / 16)];
+    };
+    auto store_stage = [&](int st) {
+#pragma unroll
+        for (int i = 0; i < 10; ++i) s_stage[st][dst[i]] = raw[i];
+    };
+    // read side: wavefront (wave & 1) takes tokens [64*(wave&1), +64), (wave >> 1) experts [32*(wave>>1), +32)
+    const int a_row0 = 64 * (wave & 1) + row;
+    const int b_row0 = BIG_TOKENS + 32 * (wave >> 1) + row;
+    auto operand = [&](int st, int r, int s) {
+        return __builtin_bit_cast(bf16x8, s_stage[st][r * 8 + ((4 * half + s) ^ ((r >> 1) & 7))]);
+    };
+
+    floatx16 acc[2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+        acc[a] = floatx16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    load_chunk(0);
+    store_stage(0);
+    __syncthreads();
+    for (int c = 0; c < n_chunks; ++c) {
+        const int st = c & 1;
+        if (c + 1 < n_chunks) load_chunk(c + 1);  // in flight under the MFMAs below
+        bf16x8 a_op[2][4];
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int s = 0; s < 4; ++s) a_op[a][s] = operand(st, a_row0 + 32 * a, s);
+        // smallest terms first
+#pragma unroll
+        for (int p = 2; p >= 0; --p) {
+            bf16x8 b_op[4];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) b_op[s] = operand(st, b_row0 + BIG_EXPERTS * p, s);
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_op[0][s], b_op[s], acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_op[1][s], b_op[s], acc[1], 0, 0, 0);
+            }
+        }
+        if (c + 1 < n_chunks) store_stage(st ^ 1);  // (last read before the barrier that ended the previous pass)
+        __syncthreads();
+    }
+    const int e = e0 + 32 * (wave >> 1) + row;
+    if (e < n_experts) {
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int tt = t0 + 64 * (wave & 1) + 32 * a + 8 * (i / 4) + 4 * half + (i % 4);
+                if (tt < tokens) out[(size_t)tt * n_experts + e] = acc[a][i];
+            }
+    }
+}
+
 // logits = partial[0] + partial[1] + ... in that order
 __global__ __launch_bounds__(256) void moe_router_reduce_kernel(const float* __restrict__ partial,
                                                                 float* __restrict__ logits,
@@ -320,7 +421,6 @@ extern "C" void moe_router_split_weight_launcher(void* planes, const float* w, i
 extern "C" void moe_router_logits_split_launcher(float* logits, const void* x, const void* planes,
                                                  void* workspace, size_t workspace_bytes, int tokens,
                                                  int hidden, int n_experts, int config, hipStream_t stream) {
-    (void)config;
     if (tokens <= 0 || n_experts <= 0) return;
     if (hidden <= 0 || hidden % K_CHUNK != 0 || (tokens + 63) / 64 > 0x7fffffff / 64 ||
         (n_experts + 63) / 64 > 65535) {
@@ -340,6 +440,15 @@ extern "C" void moe_router_logits_split_launcher(float* logits, const void* x, c
         return;
     }
     const int n_chunks = hidden / K_CHUNK;
+    // enough 128 x 64 tiles to fill the chip: the workgroup-tiled kernel (config 1 forces the other one)
+    if (splits == 1 && config != 1 &&
+        (long)((tokens + BIG_TOKENS - 1) / BIG_TOKENS) * ((n_experts + BIG_EXPERTS - 1) / BIG_EXPERTS) >= 192) {
+        const dim3 big_grid((tokens + BIG_TOKENS - 1) / BIG_TOKENS, (n_experts + BIG_EXPERTS - 1) / BIG_EXPERTS);
+        moe_router_gemm_split_tiled_kernel<<<big_grid, 256, 0, stream>>>(
+            static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(planes), logits, tokens, hidden,
+            n_experts);
+        return;
+    }
     const int chunks_per_split = (n_chunks + splits - 1) / splits;
     float* out = splits > 1 ? static_cast<float*>(workspace) : logits;
     const dim3 grid((tokens + 63) / 64, (n_experts + 63) / 64, splits);

@@ -193,7 +193,7 @@ def run_logits_split(capi, dev, x, w):
 
 
 @pytest.mark.parametrize('shape', [(64, 7168, 256), (1, 64, 32), (100, 448, 72), (700, 1024, 256), (33, 128, 1),
-                                   (130, 2048, 384)])
+                                   (130, 2048, 384), (6200, 448, 250), (12345, 64, 70)])   # the last two: workgroup-tiled kernel
 def test_split_weight_logits_match_float64(capi, dev, shape):
     T, H, E = shape
     gen = torch.Generator().manual_seed(T + E + 1)
