@@ -462,10 +462,54 @@ __global__ __launch_bounds__(1024) void moe_route_sort_small_kernel(
     }
 }
 
+// The sort of a small batch alone (tokens*slots <= 1024 pairs, one workgroup): ids come from the routing
+// kernel, which spreads the tokens over many CUs (on one CU the 8 arg-max rounds of 64 tokens are bound by
+// that CU's instruction issue rate: 24 of the 31 us the fused kernel above takes).
+__global__ __launch_bounds__(1024) void moe_sort_small_kernel(const int* __restrict__ ids,
+                                                              int* __restrict__ sorted_pairs,
+                                                              int* __restrict__ pair_pos,
+                                                              int* __restrict__ expert_offsets, int pairs,
+                                                              int sorted_experts) {
+    __shared__ int s_count[512 + 2];
+    __shared__ int s_wave_count[16][512 + 1];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int p = threadIdx.x;
+    const int mine = p < pairs ? ids[p] : -1;  // (requested before the tables are cleared)
+    for (int e = threadIdx.x; e <= sorted_experts; e += 1024) s_count[e] = 0;
+    for (int i = threadIdx.x; i < 16 * (512 + 1); i += 1024) (&s_wave_count[0][0])[i] = 0;
+    __syncthreads();
+    int rank;
+    bool later;
+    group_rank(mine, lane, rank, later);
+    if (mine >= 0 && !later) s_wave_count[wave][mine] = rank + 1;  // this wavefront's pairs of the expert
+    __syncthreads();
+    for (int e = threadIdx.x; e < sorted_experts; e += 1024) {
+        int run = 0;
+#pragma unroll
+        for (int w = 0; w < 16; ++w) {
+            const int c = s_wave_count[w][e];
+            s_wave_count[w][e] = run;
+            run += c;
+        }
+        s_count[e] = run;
+    }
+    __syncthreads();
+    if (mine >= 0) rank += s_wave_count[wave][mine];
+    block_exclusive_scan(s_count, sorted_experts);  // in place; s_count[sorted_experts] = number of pairs
+    for (int e = threadIdx.x; e <= sorted_experts; e += 1024) expert_offsets[e] = s_count[e];
+    if (p < pairs) {
+        const int pos = s_count[mine] + rank;
+        sorted_pairs[pos] = p;
+        pair_pos[p] = pos;
+    }
+}
+
 }  // namespace
 
-// Routing followed by the sort, in one launch when the batch is small (tokens*top_k <= 1024),
-// otherwise as moe_route_launcher + moe_sort_launcher. Same outputs as those two.
+// Routing followed by the sort. Small batches (tokens*top_k <= 1024): the routing kernel, then the
+// single-workgroup sort (config 2: one kernel that does both in one workgroup); otherwise
+// moe_route_launcher + moe_sort_launcher. Same outputs in every form.
 extern "C" void moe_route_sort_launcher(int* ids, float* weights, int* sorted_pairs, int* pair_pos,
                                         int* expert_offsets, int* chunk_scratch, const float* logits,
                                         int tokens, int n_experts, int top_k, int config,
@@ -577,7 +621,14 @@ extern "C" void moe_route_sort_launcher(int* ids, float* weights, int* sorted_pa
         caa::set_status(CAA_BAD_ARGUMENT);
         return;
     }
-    if ((long)tokens * (top_k + shared) <= 1024 && config != 1) {
+    if ((long)tokens * (top_k + shared) <= 1024 && config != 1 && config != 2) {
+        // two launches: routing over many CUs, then the single-workgroup sort (config 2: the fused kernel)
+        moe_route_launcher(ids, weights, logits, tokens, n_experts, top_k, shared ? CONFIG_SHARED_SLOT : 0, stream);
+        moe_sort_small_kernel<<<1, 1024, 0, stream>>>(ids, sorted_pairs, pair_pos, expert_offsets,
+                                                      tokens * (top_k + shared), n_experts + shared);
+        return;
+    }
+    if ((long)tokens * (top_k + shared) <= 1024 && config == 2) {
         if (n_experts <= 256) {
             moe_route_sort_small_kernel<4><<<1, 1024, 0, stream>>>(
                 logits, ids, weights, sorted_pairs, pair_pos, expert_offsets, tokens, n_experts, top_k,

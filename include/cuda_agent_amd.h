@@ -317,8 +317,9 @@ void moe_sort_launcher(int* sorted_pairs, int* pair_pos, int* expert_offsets, in
                        const int* ids, int tokens, int n_experts, int top_k, int config,
                        hipStream_t stream);
 
-/* moe_route_launcher followed by moe_sort_launcher, as one kernel when tokens*top_k <= 1024 (the
- * decode case); same outputs. config 1 forces the two-step path. */
+/* moe_route_launcher followed by the sort; same outputs. With tokens*top_k <= 1024 (the decode case) the sort is
+ * one single-workgroup kernel behind the routing kernel; config 1 forces the chunked sort, config 2 a single
+ * kernel that routes and sorts in one workgroup. */
 void moe_route_sort_launcher(int* ids, float* weights, int* sorted_pairs, int* pair_pos,
                              int* expert_offsets, int* chunk_scratch, const float* logits, int tokens,
                              int n_experts, int top_k, int config, hipStream_t stream);
