@@ -38,6 +38,23 @@ __device__ __forceinline__ uint32_t score_key(float x) {
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
+// Inclusive prefix sum over the lanes of a wavefront: running sums inside each row of 16 lanes on DPP row
+// shifts (vector ALU; the __shfl_up form is six dependent trips through the LDS crossbar), then the totals of
+// the rows before a lane's own, read as scalars.
+__device__ __forceinline__ int wave_inclusive_sum(int v, int lane) {
+#define ROW_SHR_ADD(n) v += __builtin_amdgcn_update_dpp(0, v, 0x110 + (n), 0xf, 0xf, false);
+    ROW_SHR_ADD(1)
+    ROW_SHR_ADD(2)
+    ROW_SHR_ADD(4)
+    ROW_SHR_ADD(8)
+#undef ROW_SHR_ADD
+    const int r0 = __builtin_amdgcn_readlane(v, 15);
+    const int r1 = __builtin_amdgcn_readlane(v, 31);
+    const int r2 = __builtin_amdgcn_readlane(v, 47);
+    const int row = lane >> 4;
+    return v + (row >= 1 ? r0 : 0) + (row >= 2 ? r1 : 0) + (row >= 3 ? r2 : 0);
+}
+
 __global__ __launch_bounds__(SELECT_THREADS) void topk_select_kernel(
     const float* __restrict__ scores, const int* __restrict__ lengths, int* __restrict__ idx_out,
     int n, int k) {
@@ -194,6 +211,11 @@ __global__ __launch_bounds__(SELECT_THREADS) void topk_select_regs_kernel(
     }
 #pragma unroll
     for (int j = 0; j < P; ++j) live |= (first + j < valid ? 1u : 0u) << j;
+    // Entries that are no candidates get the smallest key: the passes below then need no test of `live`
+    // (such an entry lands in the lowest bin of every digit, below the `want` largest live keys, or among
+    // the ties of key 0, of which the emission takes live ones only).
+#pragma unroll
+    for (int j = 0; j < P; ++j) key[j] = ((live >> j) & 1u) ? key[j] : 0u;
 
     if (tid == 0) {
         s_prefix = 0u;
@@ -206,10 +228,15 @@ __global__ __launch_bounds__(SELECT_THREADS) void topk_select_regs_kernel(
         __syncthreads();
         const uint32_t prefix = s_prefix;
         const uint32_t prefix_mask = pass == 0 ? 0u : 0xffffffffu << (shift + 8);
+        if (pass == 0) {
 #pragma unroll
-        for (int j = 0; j < P; ++j) {
-            if (((live >> j) & 1u) && (key[j] & prefix_mask) == prefix)
-                atomicAdd(&s_hist[((key[j] >> shift) & 255u) * HIST_COPIES + copy], 1);
+            for (int j = 0; j < P; ++j) atomicAdd(&s_hist[(key[j] >> 24) * HIST_COPIES + copy], 1);
+        } else {
+#pragma unroll
+            for (int j = 0; j < P; ++j) {
+                if ((key[j] & prefix_mask) == prefix)
+                    atomicAdd(&s_hist[((key[j] >> shift) & 255u) * HIST_COPIES + copy], 1);
+            }
         }
         __syncthreads();
         if (wave == 0) {
@@ -223,13 +250,7 @@ __global__ __launch_bounds__(SELECT_THREADS) void topk_select_regs_kernel(
                 for (int h = 0; h < HIST_COPIES; ++h) c[j] += s_hist[bin * HIST_COPIES + h];
                 mine += c[j];
             }
-            int above = mine;
-#pragma unroll
-            for (int d = 1; d < 64; d <<= 1) {
-                const int v = __shfl_up(above, d);
-                if (lane >= d) above += v;
-            }
-            above -= mine;
+            int above = wave_inclusive_sum(mine, lane) - mine;
             const int remaining = s_remaining;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -254,16 +275,9 @@ __global__ __launch_bounds__(SELECT_THREADS) void topk_select_regs_kernel(
             n_eq += (on && key[j] == threshold) ? 1 : 0;
         }
         // exclusive scan of (n_gt, n_eq) over the 1024 lanes, in lane order = index order
-        int gt_before = n_gt, eq_before = n_eq;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            const int g = __shfl_up(gt_before, d);
-            const int e = __shfl_up(eq_before, d);
-            if (lane >= d) {
-                gt_before += g;
-                eq_before += e;
-            }
-        }
+        // (both counts fit 16 bits: one scan of the packed pair)
+        const int packed_before = wave_inclusive_sum(n_gt | (n_eq << 16), lane);
+        int gt_before = packed_before & 0xffff, eq_before = packed_before >> 16;
         if (lane == 63) {
             s_wave_gt[wave] = gt_before;
             s_wave_eq[wave] = eq_before;
