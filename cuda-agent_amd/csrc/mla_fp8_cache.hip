@@ -30,6 +30,12 @@ extern "C" void sparse_mla_decode_launcher(void* out, const void* q, const void*
                                            void* workspace, size_t workspace_bytes, int batch,
                                            int n_heads, int n_kv_rows, int topk, int d_qk, int d_v,
                                            float sm_scale, int out_dtype, int config, hipStream_t stream);
+extern "C" int sparse_mla_decode_fp8_fused(void* out, const void* q, const void* kv_fp8, const int* idx,
+                                           void* workspace, size_t workspace_bytes, int batch, int n_heads,
+                                           int n_kv_rows, int topk, int d_qk, int d_v, float sm_scale,
+                                           int out_dtype, int config, const int* block_table,
+                                           int table_stride, int page_shift, int batch_rows,
+                                           hipStream_t stream);
 
 namespace {
 
@@ -186,6 +192,7 @@ extern "C" void mla_latent_quant_launcher(void* cache, const void* kv, long rows
 // compact block of dequantised rows and its index list
 extern "C" size_t sparse_mla_decode_fp8_workspace_bytes(int batch, int n_heads, int topk, int config) {
     if (batch <= 0 || n_heads <= 0 || topk <= 0) return 0;
+    if (config >= 5000) config -= 5000;
     return align16(sparse_mla_decode_workspace_bytes(batch, n_heads, topk, config)) +
            align16((size_t)batch * topk * ROW_BF16_BYTES) + align16((size_t)batch * topk * sizeof(int));
 }
@@ -210,7 +217,16 @@ void launch_decode_fp8(void* out, const void* q, const void* kv_fp8, const int* 
         caa::set_status(CAA_WORKSPACE_TOO_SMALL);
         return;
     }
+    // config 5000 + n: the two-step form (gather + dequantise into the workspace, then the bf16 kernels) with
+    // config n; otherwise the 128-head kernel dequantises its tiles itself where the shape allows
+    const bool two_step = config >= 5000;
+    if (two_step) config -= 5000;
     const size_t base_bytes = align16(sparse_mla_decode_workspace_bytes(batch, n_heads, topk, config));
+    if (!two_step &&
+        sparse_mla_decode_fp8_fused(out, q, kv_fp8, idx, workspace, base_bytes, batch, n_heads, n_kv_rows, topk,
+                                    d_qk, d_v, sm_scale, out_dtype, config, kva.block_table, kva.table_stride,
+                                    kva.page_shift, kva.batch_rows, stream))
+        return;
     uint8_t* ws = static_cast<uint8_t*>(workspace);
     __hip_bfloat16* rows = reinterpret_cast<__hip_bfloat16*>(ws + base_bytes);
     int* compact_idx = reinterpret_cast<int*>(ws + base_bytes + align16((size_t)batch * topk * ROW_BF16_BYTES));

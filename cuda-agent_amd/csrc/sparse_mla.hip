@@ -536,7 +536,81 @@ __device__ __forceinline__ void gather_issue(uint4* tile, const char* kv_b, uint
     }
 }
 
-// grid: x = split, y = request, z = group of 128 heads; 512 lanes
+// ---- e4m3 storage form of the cache (rows of 656 bytes: 512 codes, 4 fp32 scales, 64 bf16 rope values) ----
+// The 41 chunks of such a row are DMA'd to positions 31..71 of the row's own 72-chunk tile row: codes and
+// scales as they come (positions 31..63), the rope chunks straight to their final, swizzled positions
+// 64..71. The wavefront that gathered the row then reads codes and scales into registers and writes the 64
+// chunks of bf16 latent values over positions 0..63 (a wavefront's LDS operations execute in order, and every
+// read of the row is issued before its first write). No LDS beyond the tile ring is needed.
+constexpr int FP8_ROW_BYTES = 656;
+constexpr int FP8_ROW_CHUNKS = FP8_ROW_BYTES / 16;  // 41
+constexpr int FP8_FIRST_SLOT = ROW_CHUNKS - FP8_ROW_CHUNKS;  // 31
+constexpr int FP8_GATHER_INSTR = 8;  // one load instruction per row of a wavefront's quarter
+
+// row i (0..7) of quarter `quarter` of a tile; key < 0: padding, the row is zero-filled
+__device__ __forceinline__ void gather_issue_fp8(uint4* tile, const char* kv_b, int key, int i, int quarter,
+                                                 int lane) {
+    // (the lane number is hidden from the optimiser: the per-row chunk numbers would otherwise be precomputed
+    // for all eight rows outside the tile loop, spilled, and every reload would wait for all loads in flight)
+    asm volatile("" : "+v"(lane));
+    const int row = 8 * quarter + i;
+    uint4* slots = tile + row * ROW_CHUNKS;
+    if (key >= 0) {
+        if (lane < FP8_ROW_CHUNKS) {
+            // lanes 0..32: codes and scales; lanes 33..40: the rope chunk that belongs at position 31 + lane
+            const int chunk = lane < 33 ? lane : 33 + (((lane - 33) ^ row_swizzle(row)) & 7);
+            const uint32_t off = (uint32_t)key * (uint32_t)FP8_ROW_BYTES + 16u * (uint32_t)chunk;
+            const uint32_t lds_base = (uint32_t)(size_t)((lds_void_ptr)(slots + FP8_FIRST_SLOT));
+            asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+                         :
+                         : "v"(off), "s"(kv_b), "s"(lds_base)
+                         : "memory", "m0");
+        }
+    } else {
+        slots[lane] = make_uint4(0u, 0u, 0u, 0u);
+        if (lane < ROW_CHUNKS - 64) slots[64 + lane] = make_uint4(0u, 0u, 0u, 0u);
+    }
+}
+
+// two e4m3 codes (one half of a dword) times a scale -> two bf16 (round to nearest even) in one dword
+__device__ __forceinline__ uint32_t dequant_pair(uint32_t codes, bool upper, float scale) {
+    typedef float floatx2 __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    const floatx2 f = upper ? __builtin_amdgcn_cvt_pk_f32_fp8((int)codes, true)
+                            : __builtin_amdgcn_cvt_pk_f32_fp8((int)codes, false);
+    const bf16x2 r = {(__bf16)(f[0] * scale), (__bf16)(f[1] * scale)};
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+// the 8 rows of quarter `quarter`: codes and scales at positions 31..63 -> bf16 latent values at 0..63. Two
+// rows at a time: lanes 0-31 take row 2*j, lanes 32-63 row 2*j + 1; a lane converts 16 codes and reads the
+// scale of its block of 128 straight from the row's scale chunk.
+__device__ __forceinline__ void dequant_quarter(uint4* tile, const int* s_idx_tile, int quarter, int lane) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        asm volatile("" : "+v"(lane));  // (as in gather_issue_fp8: no per-row addresses kept across the tile loop)
+        const int sub = lane & 31;
+        const int x = 2 * sub;  // bf16 chunks 2*sub and 2*sub + 1 of the row
+        const int row = 8 * quarter + 2 * j + (lane >> 5);
+        uint4* slots = tile + row * ROW_CHUNKS;
+        const bool live = s_idx_tile[row] >= 0;  // (a padding row was zero-filled by the gather)
+        const uint4 c = slots[FP8_FIRST_SLOT + sub];
+        const float sc = reinterpret_cast<const float*>(slots + FP8_FIRST_SLOT + 32)[sub >> 3];
+        const int swz = row_swizzle(row);
+        if (live) {
+            slots[(x & ~7) | ((x ^ swz) & 7)] =
+                make_uint4(dequant_pair(c.x, false, sc), dequant_pair(c.x, true, sc), dequant_pair(c.y, false, sc),
+                           dequant_pair(c.y, true, sc));
+            slots[(x & ~7) | (((x + 1) ^ swz) & 7)] =
+                make_uint4(dequant_pair(c.z, false, sc), dequant_pair(c.z, true, sc), dequant_pair(c.w, false, sc),
+                           dequant_pair(c.w, true, sc));
+        }
+        __builtin_amdgcn_sched_barrier(0);  // one pair of rows at a time: registers are short here
+    }
+}
+
+// grid: x = split, y = request, z = group of 128 heads; 512 lanes. FP8: kv is a cache in the 656-byte e4m3 form.
+template <bool FP8>
 __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ kv, const int* __restrict__ idx,
     _Float16* __restrict__ o_part, float* __restrict__ lse_part, float* __restrict__ scale_part,
@@ -621,19 +695,27 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
     }
     __syncthreads();
     const int first_masked_tile = s_first_masked_tile;
-    const char* kv_b = reinterpret_cast<const char*>(kv) + (size_t)b * kva.batch_rows * ROW_BYTES;
+    const char* kv_b = reinterpret_cast<const char*>(kv) + (size_t)b * kva.batch_rows * (FP8 ? FP8_ROW_BYTES : ROW_BYTES);
     PHASE_MARK(7);  // index staging
 
     // The first two tiles are on their way before Q is fetched: tile 0 by the lead group, tile 1
     // by the lag group (a cold load instruction takes several hundred cycles to issue, so the
     // two groups share the work; from tile 2 on the lag group gathers alone).
     if (group < n_tiles) {
-        uint32_t off[GATHER_INSTR];
-        const bool pad = group >= first_masked_tile;
-        gather_prepare(off, s_idx + group * TILE_ROWS, s_gather_tab, pad, wave & 3, lane);
+        if constexpr (FP8) {
 #pragma unroll
-        for (int i = 0; i < GATHER_INSTR; ++i) {
-            gather_issue(tiles + group * TILE_CHUNKS, kv_b, off[i], i, pad, wave & 3, lane);
+            for (int i = 0; i < FP8_GATHER_INSTR; ++i) {
+                const int key = __builtin_amdgcn_readfirstlane(s_idx[group * TILE_ROWS + 8 * (wave & 3) + i]);
+                gather_issue_fp8(tiles + group * TILE_CHUNKS, kv_b, key, i, wave & 3, lane);
+            }
+        } else {
+            uint32_t off[GATHER_INSTR];
+            const bool pad = group >= first_masked_tile;
+            gather_prepare(off, s_idx + group * TILE_ROWS, s_gather_tab, pad, wave & 3, lane);
+#pragma unroll
+            for (int i = 0; i < GATHER_INSTR; ++i) {
+                gather_issue(tiles + group * TILE_CHUNKS, kv_b, off[i], i, pad, wave & 3, lane);
+            }
         }
     }
     PHASE_MARK(9);  // first gather issue
@@ -689,11 +771,18 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
         if ((h & 1) == 0 && h < 2 * n_tiles) {
             // tile h/2 must be resident: everything but this wavefront's share of the next tile
             const int t = h >> 1;
-            const bool plain_wait = t + 1 < n_tiles && t + 1 < first_masked_tile;
+            const bool plain_wait = t + 1 < n_tiles && t + 1 < first_masked_tile && !(FP8 && h == 0);
             if (plain_wait) {
-                wait_vmcnt<GATHER_INSTR>();  // (the lead group has no loads in flight)
+                wait_vmcnt<FP8 ? FP8_GATHER_INSTR : GATHER_INSTR>();  // (the lead group has no loads in flight)
             } else {
                 wait_all_memory();
+            }
+            if constexpr (FP8) {
+                // the wavefronts that gathered tile t (the lead group for tile 0, the lag group otherwise) turn
+                // its rows into bf16 before the barrier below hands the tile to everyone
+                asm volatile("" ::: "memory");  // the reads below stay behind the wait above
+                if (group == (t == 0 ? 0 : 1))
+                    dequant_quarter(tiles + (t % 3) * TILE_CHUNKS, s_idx + t * TILE_ROWS, wave & 3, lane);
             }
         }
         __builtin_amdgcn_s_waitcnt((63 & 15) | ((63 >> 4) << 14) | (7 << 4) | (0 << 8));  // lgkmcnt(0)
@@ -719,11 +808,19 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
             // at one per ~150 cycles whether or not MFMAs are issued in between (measured), so
             // they go out back to back and the QK^T loop stays free of them.
             if (gather) {
-                uint32_t goff[GATHER_INSTR];
-                gather_prepare(goff, s_idx + t2 * TILE_ROWS, s_gather_tab, gather_pad, wave & 3, lane);
+                if constexpr (FP8) {
 #pragma unroll
-                for (int i = 0; i < GATHER_INSTR; ++i) {
-                    gather_issue(gather_tile, kv_b, goff[i], i, gather_pad, wave & 3, lane);
+                    for (int i = 0; i < FP8_GATHER_INSTR; ++i) {
+                        const int key = __builtin_amdgcn_readfirstlane(s_idx[t2 * TILE_ROWS + 8 * (wave & 3) + i]);
+                        gather_issue_fp8(gather_tile, kv_b, key, i, wave & 3, lane);
+                    }
+                } else {
+                    uint32_t goff[GATHER_INSTR];
+                    gather_prepare(goff, s_idx + t2 * TILE_ROWS, s_gather_tab, gather_pad, wave & 3, lane);
+#pragma unroll
+                    for (int i = 0; i < GATHER_INSTR; ++i) {
+                        gather_issue(gather_tile, kv_b, goff[i], i, gather_pad, wave & 3, lane);
+                    }
                 }
             }
             PHASE_MARK(2);  // gather issue
@@ -993,10 +1090,12 @@ namespace {
 
 // shared by the two launchers: n_kv_rows is the number of rows of the block a request's keys
 // resolve into (the request's own cache, or the whole pool)
+// fp8_cache: kv is in the 656-byte e4m3 form, which only the 128-head kernel reads (the caller has checked
+// the shape with fp8_cache_fused_ok)
 void launch_sparse_mla(void* out, const void* q, const void* kv, const int* idx, void* workspace,
                        size_t workspace_bytes, int batch, int n_heads, int n_kv_rows, int topk,
                        int d_qk, int d_v, float sm_scale, int out_dtype, int config,
-                       const KvAddressing& kva, hipStream_t stream) {
+                       const KvAddressing& kva, hipStream_t stream, bool fp8_cache = false) {
     if (batch <= 0 || n_heads <= 0 || topk <= 0) return;
     const bool heads_ok = n_heads == 32 || n_heads == 64 || (n_heads % 128 == 0);
     if (d_qk != D_QK || d_v != D_V || !heads_ok || n_kv_rows <= 0 || batch > 65535 ||
@@ -1019,7 +1118,8 @@ void launch_sparse_mla(void* out, const void* q, const void* kv, const int* idx,
     // split count)
     // The 8-wavefront kernel addresses a request's cache block with 32-bit byte offsets.
     const bool four_wave_kernel =
-        config >= 1000 || (unsigned long long)n_kv_rows * ROW_BYTES >= 0xffffffffull;
+        config >= 1000 ||
+        (unsigned long long)n_kv_rows * (fp8_cache ? FP8_ROW_BYTES : ROW_BYTES) >= 0xffffffffull;
     if (config >= 1000) config -= 1000;
     const int head_groups = n_heads <= 128 ? 1 : n_heads / 128;
     const int splits = pick_splits(batch, head_groups, topk, config);
@@ -1048,9 +1148,15 @@ void launch_sparse_mla(void* out, const void* q, const void* kv, const int* idx,
                                                              scale_log2, kva);
     } else {
         half_parts = true;  // this kernel stores its partials as scaled fp16
-        sparse_mla_split8_kernel<<<grid, 512, 0, stream>>>(
-            qb, kvb, idx, reinterpret_cast<_Float16*>(o_part), lse_part, scale_part, n_heads, n_kv_rows,
-            topk, rows_per_split, scale_log2, kva);
+        if (fp8_cache) {
+            sparse_mla_split8_kernel<true><<<grid, 512, 0, stream>>>(
+                qb, kvb, idx, reinterpret_cast<_Float16*>(o_part), lse_part, scale_part, n_heads, n_kv_rows,
+                topk, rows_per_split, scale_log2, kva);
+        } else {
+            sparse_mla_split8_kernel<false><<<grid, 512, 0, stream>>>(
+                qb, kvb, idx, reinterpret_cast<_Float16*>(o_part), lse_part, scale_part, n_heads, n_kv_rows,
+                topk, rows_per_split, scale_log2, kva);
+        }
     }
     // rows requested at once per lane: as many as there are splits, up to 8
 #define MLA_MERGE(OUT_T, PART_T, PARTS, SCALES)                                                   \
@@ -1130,4 +1236,24 @@ extern "C" void sparse_mla_decode_paged_launcher(void* out, const void* q, const
     const KvAddressing kva{block_table, max_pages_per_request, page_shift, 0};
     launch_sparse_mla(out, q, kv_pool, idx, workspace, workspace_bytes, batch, n_heads,
                       n_pages * page_size, topk, d_qk, d_v, sm_scale, out_dtype, config, kva, stream);
+}
+
+// Decode over a cache in the 656-byte e4m3 form with the dequantisation inside the 128-head kernel (see
+// gather_issue_fp8 / dequant_quarter). Returns 1 if the launch was made (or rejected with a status), 0 if
+// this shape has to take the two-step form of sparse_mla_decode_fp8_launcher: head counts other than
+// multiples of 128, config >= 1000, caches of 4 GB and more per addressed block.
+// block_table / table_stride / page_shift / batch_rows: the addressing of the cache, as in KvAddressing.
+extern "C" int sparse_mla_decode_fp8_fused(void* out, const void* q, const void* kv_fp8, const int* idx,
+                                           void* workspace, size_t workspace_bytes, int batch, int n_heads,
+                                           int n_kv_rows, int topk, int d_qk, int d_v, float sm_scale,
+                                           int out_dtype, int config, const int* block_table,
+                                           int table_stride, int page_shift, int batch_rows,
+                                           hipStream_t stream) {
+    if (n_heads <= 0 || n_heads % 128 != 0 || config >= 1000 || n_kv_rows <= 0 ||
+        (unsigned long long)n_kv_rows * FP8_ROW_BYTES >= 0xffffffffull)
+        return 0;
+    const KvAddressing kva{block_table, table_stride, page_shift, batch_rows};
+    launch_sparse_mla(out, q, kv_fp8, idx, workspace, workspace_bytes, batch, n_heads, n_kv_rows, topk, d_qk,
+                      d_v, sm_scale, out_dtype, config, kva, stream, true);
+    return 1;
 }

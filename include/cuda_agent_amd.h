@@ -177,10 +177,13 @@ void mla_latent_quant_launcher(void* cache, const void* kv, long rows, int confi
  * block [batch, topk, 576] bf16 of dequantised selected rows and its index list. */
 size_t sparse_mla_decode_fp8_workspace_bytes(int batch, int n_heads, int topk, int config);
 
-/* sparse_mla_decode_launcher over kv_fp8 [batch, n_kv_rows, 656] bytes in the form above: the selected rows
- * are gathered and dequantised (code * scale in fp32, rounded to nearest-even bf16) into the workspace, then
- * attended as by sparse_mla_decode_launcher; the result equals that launcher's on the dequantised cache
- * bit for bit. Other arguments, limits and config as there. */
+/* sparse_mla_decode_launcher over kv_fp8 [batch, n_kv_rows, 656] bytes in the form above. Each selected row is
+ * dequantised as code * scale in fp32, rounded to nearest-even bf16, and attended as by
+ * sparse_mla_decode_launcher: the result equals that launcher's on the dequantised cache bit for bit. With
+ * n_heads a multiple of 128, config below 1000 and a cache below 4 GB per request the split kernel gathers the
+ * 656-byte rows itself and dequantises every key tile in LDS; otherwise, or with 5000 added to config, the
+ * selected rows are first dequantised into the workspace and the bf16 kernels run on that block (same bits).
+ * Other arguments, limits and config as sparse_mla_decode_launcher. */
 void sparse_mla_decode_fp8_launcher(void* out, const void* q, const void* kv_fp8, const int* idx,
                                     void* workspace, size_t workspace_bytes, int batch, int n_heads,
                                     int n_kv_rows, int topk, int d_qk, int d_v, float sm_scale,

@@ -66,6 +66,8 @@ def test_decode_over_the_fp8_cache(capi, dev, shape):
     deq = mla.latent_dequantize(cache.cpu())
     assert torch.equal(got32, run_bf16(capi, dev, q, deq, idx, torch.float32))
     assert torch.equal(run_fp8(capi, dev, q, cache, idx), run_bf16(capi, dev, q, deq, idx))
+    # config 5000+n asks for the two-step form (dequantise into the workspace, then the bf16 kernels): same bits
+    assert torch.equal(run_fp8(capi, dev, q, cache, idx, torch.float32, config=5000), got32)
     # and not far from the attention over the unquantised rows (e4m3 keeps 3 mantissa bits)
     exact = mla.sparse_mla_decode(q, kv, idx, out_dtype=torch.float32)
     assert ((got32 - exact).pow(2).mean().sqrt() / exact.pow(2).mean().sqrt()).item() <= 0.1
@@ -78,6 +80,7 @@ def test_all_padding_and_forced_splits(capi, dev):
     idx[1] = -1                               # a request without any selected row: zeros
     out = run_fp8(capi, dev, q, cache, idx, torch.float32, config=3)
     assert (out[1] == 0).all()
+    assert torch.equal(run_fp8(capi, dev, q, cache, idx, torch.float32, config=5003), out)
     ref = mla.sparse_mla_decode_fp8(q[:1], cache[:1], idx[:1], out_dtype=torch.float32)
     assert mla.rel_rms_error(out[:1], ref) <= TOL
 
