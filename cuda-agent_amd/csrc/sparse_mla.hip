@@ -583,30 +583,36 @@ __device__ __forceinline__ uint32_t dequant_pair(uint32_t codes, bool upper, flo
 }
 
 // the 8 rows of quarter `quarter`: codes and scales at positions 31..63 -> bf16 latent values at 0..63. Two
-// rows at a time: lanes 0-31 take row 2*j, lanes 32-63 row 2*j + 1; a lane converts 16 codes and reads the
-// scale of its block of 128 straight from the row's scale chunk.
-__device__ __forceinline__ void dequant_quarter(uint4* tile, const int* s_idx_tile, int quarter, int lane) {
+// rows per step: lanes 0-31 take row 2*j, lanes 32-63 row 2*j + 1; a lane converts 16 codes and reads the
+// scale of its block of 128 straight from the row's scale chunk. All reads of the quarter are issued before the
+// first write (a wavefront's LDS operations execute in order, and the quarter belongs to this wavefront alone).
+// A padding row was zero-filled by the gather: codes 0 times scale 0 writes the same zeros again.
+__device__ __forceinline__ void dequant_quarter(uint4* tile, int quarter, int lane) {
+    asm volatile("" : "+v"(lane));  // (as in gather_issue_fp8: no per-row addresses kept across the tile loop)
+    const int sub = lane & 31;
+    const int x = 2 * sub;  // bf16 chunks 2*sub and 2*sub + 1 of the row
+    uint4* slots0 = tile + (8 * quarter + (lane >> 5)) * ROW_CHUNKS;
+    uint4 c[4];
+    float sc[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        asm volatile("" : "+v"(lane));  // (as in gather_issue_fp8: no per-row addresses kept across the tile loop)
-        const int sub = lane & 31;
-        const int x = 2 * sub;  // bf16 chunks 2*sub and 2*sub + 1 of the row
-        const int row = 8 * quarter + 2 * j + (lane >> 5);
-        uint4* slots = tile + row * ROW_CHUNKS;
-        const bool live = s_idx_tile[row] >= 0;  // (a padding row was zero-filled by the gather)
-        const uint4 c = slots[FP8_FIRST_SLOT + sub];
-        const float sc = reinterpret_cast<const float*>(slots + FP8_FIRST_SLOT + 32)[sub >> 3];
-        const int swz = row_swizzle(row);
-        if (live) {
-            slots[(x & ~7) | ((x ^ swz) & 7)] =
-                make_uint4(dequant_pair(c.x, false, sc), dequant_pair(c.x, true, sc), dequant_pair(c.y, false, sc),
-                           dequant_pair(c.y, true, sc));
-            slots[(x & ~7) | (((x + 1) ^ swz) & 7)] =
-                make_uint4(dequant_pair(c.z, false, sc), dequant_pair(c.z, true, sc), dequant_pair(c.w, false, sc),
-                           dequant_pair(c.w, true, sc));
-        }
-        __builtin_amdgcn_sched_barrier(0);  // one pair of rows at a time: registers are short here
+        const uint4* slots = slots0 + 2 * j * ROW_CHUNKS;
+        c[j] = slots[FP8_FIRST_SLOT + sub];
+        sc[j] = reinterpret_cast<const float*>(slots + FP8_FIRST_SLOT + 32)[sub >> 3];
     }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        uint4* slots = slots0 + 2 * j * ROW_CHUNKS;
+        const int swz = row_swizzle(8 * quarter + 2 * j + (lane >> 5));
+        slots[(x & ~7) | ((x ^ swz) & 7)] =
+            make_uint4(dequant_pair(c[j].x, false, sc[j]), dequant_pair(c[j].x, true, sc[j]),
+                       dequant_pair(c[j].y, false, sc[j]), dequant_pair(c[j].y, true, sc[j]));
+        slots[(x & ~7) | (((x + 1) ^ swz) & 7)] =
+            make_uint4(dequant_pair(c[j].z, false, sc[j]), dequant_pair(c[j].z, true, sc[j]),
+                       dequant_pair(c[j].w, false, sc[j]), dequant_pair(c[j].w, true, sc[j]));
+    }
+    __builtin_amdgcn_sched_barrier(0);
 }
 
 // grid: x = split, y = request, z = group of 128 heads; 512 lanes. FP8: kv is a cache in the 656-byte e4m3 form.
@@ -703,10 +709,10 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
     // two groups share the work; from tile 2 on the lag group gathers alone).
     if (group < n_tiles) {
         if constexpr (FP8) {
+            const int keys = s_idx[group * TILE_ROWS + 8 * (wave & 3) + (lane & 7)];  // one LDS read for the 8 rows
 #pragma unroll
             for (int i = 0; i < FP8_GATHER_INSTR; ++i) {
-                const int key = __builtin_amdgcn_readfirstlane(s_idx[group * TILE_ROWS + 8 * (wave & 3) + i]);
-                gather_issue_fp8(tiles + group * TILE_CHUNKS, kv_b, key, i, wave & 3, lane);
+                gather_issue_fp8(tiles + group * TILE_CHUNKS, kv_b, __builtin_amdgcn_readlane(keys, i), i, wave & 3, lane);
             }
         } else {
             uint32_t off[GATHER_INSTR];
@@ -782,7 +788,7 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
                 // its rows into bf16 before the barrier below hands the tile to everyone
                 asm volatile("" ::: "memory");  // the reads below stay behind the wait above
                 if (group == (t == 0 ? 0 : 1))
-                    dequant_quarter(tiles + (t % 3) * TILE_CHUNKS, s_idx + t * TILE_ROWS, wave & 3, lane);
+                    dequant_quarter(tiles + (t % 3) * TILE_CHUNKS, wave & 3, lane);
             }
         }
         __builtin_amdgcn_s_waitcnt((63 & 15) | ((63 >> 4) << 14) | (7 << 4) | (0 << 8));  // lgkmcnt(0)
@@ -809,10 +815,10 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
             // they go out back to back and the QK^T loop stays free of them.
             if (gather) {
                 if constexpr (FP8) {
+                    const int keys = s_idx[t2 * TILE_ROWS + 8 * (wave & 3) + (lane & 7)];
 #pragma unroll
                     for (int i = 0; i < FP8_GATHER_INSTR; ++i) {
-                        const int key = __builtin_amdgcn_readfirstlane(s_idx[t2 * TILE_ROWS + 8 * (wave & 3) + i]);
-                        gather_issue_fp8(gather_tile, kv_b, key, i, wave & 3, lane);
+                        gather_issue_fp8(gather_tile, kv_b, __builtin_amdgcn_readlane(keys, i), i, wave & 3, lane);
                     }
                 } else {
                     uint32_t goff[GATHER_INSTR];
