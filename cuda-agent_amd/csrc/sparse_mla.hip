@@ -537,38 +537,43 @@ __device__ __forceinline__ void gather_issue(uint4* tile, const char* kv_b, uint
 }
 
 // ---- e4m3 storage form of the cache (rows of 656 bytes: 512 codes, 4 fp32 scales, 64 bf16 rope values) ----
-// The 41 chunks of such a row are DMA'd to positions 31..71 of the row's own 72-chunk tile row: codes and
-// scales as they come (positions 31..63), the rope chunks straight to their final, swizzled positions
-// 64..71. The wavefront that gathered the row then reads codes and scales into registers and writes the 64
-// chunks of bf16 latent values over positions 0..63 (a wavefront's LDS operations execute in order, and every
-// read of the row is issued before its first write). No LDS beyond the tile ring is needed.
+// A wavefront gathers the 8 rows of its quarter of a tile as 328 consecutive 16-byte chunks (row r at chunks
+// 41*r .. 41*r + 40) at the start of the quarter's own region of the tile, with 6 load instructions of 64 lanes
+// (the last one of 8): a load instruction costs the same to issue whether 41 or 64 of its lanes fetch. The same
+// wavefront then reads all of it into registers (4 code chunks, their scales and one rope chunk per lane) and
+// writes the 8 rows in the tile's bf16 layout over the region (a wavefront's LDS operations execute in order, and
+// every read is issued before the first write). No LDS beyond the tile ring is needed.
 constexpr int FP8_ROW_BYTES = 656;
 constexpr int FP8_ROW_CHUNKS = FP8_ROW_BYTES / 16;  // 41
-constexpr int FP8_FIRST_SLOT = ROW_CHUNKS - FP8_ROW_CHUNKS;  // 31
-constexpr int FP8_GATHER_INSTR = 8;  // one load instruction per row of a wavefront's quarter
+constexpr int FP8_STAGE_CHUNKS = 8 * FP8_ROW_CHUNKS;  // 328 chunks of a quarter
+constexpr int FP8_GATHER_INSTR = (FP8_STAGE_CHUNKS + 63) / 64;  // 6
 
-// row i (0..7) of quarter `quarter` of a tile; key < 0: padding, the row is zero-filled
-__device__ __forceinline__ void gather_issue_fp8(uint4* tile, const char* kv_b, int key, int i, int quarter,
-                                                 int lane) {
-    // (the lane number is hidden from the optimiser: the per-row chunk numbers would otherwise be precomputed
-    // for all eight rows outside the tile loop, spilled, and every reload would wait for all loads in flight)
+// quarter `quarter` of a tile. pad: the tile has padding entries (key < 0): their lanes fetch row 0, and the
+// dequantisation writes zeros for them.
+__device__ __forceinline__ void gather_quarter_fp8(uint4* tile, const char* kv_b, const int* s_idx_tile, bool pad,
+                                                   int quarter, int lane) {
+    // (the lane number is hidden from the optimiser: per-lane row and chunk numbers would otherwise be kept
+    // across the tile loop, spilled, and a scratch reload in front of a load waits for all loads in flight)
     asm volatile("" : "+v"(lane));
-    const int row = 8 * quarter + i;
-    uint4* slots = tile + row * ROW_CHUNKS;
-    if (key >= 0) {
-        if (lane < FP8_ROW_CHUNKS) {
-            // lanes 0..32: codes and scales; lanes 33..40: the rope chunk that belongs at position 31 + lane
-            const int chunk = lane < 33 ? lane : 33 + (((lane - 33) ^ row_swizzle(row)) & 7);
-            const uint32_t off = (uint32_t)key * (uint32_t)FP8_ROW_BYTES + 16u * (uint32_t)chunk;
-            const uint32_t lds_base = (uint32_t)(size_t)((lds_void_ptr)(slots + FP8_FIRST_SLOT));
+    uint32_t off[FP8_GATHER_INSTR];
+#pragma unroll
+    for (int k = 0; k < FP8_GATHER_INSTR; ++k) {
+        const int g = 64 * k + lane;       // chunk of the quarter
+        int r = (g * 25) >> 10;            // g / 41 for g < 328
+        r = r > 7 ? 7 : r;                 // (idle lanes of the last instruction)
+        int key = s_idx_tile[8 * quarter + r];
+        if (pad) key = key < 0 ? 0 : key;
+        off[k] = (uint32_t)key * (uint32_t)FP8_ROW_BYTES + 16u * (uint32_t)(g - FP8_ROW_CHUNKS * r);
+    }
+    const uint32_t lds_base = (uint32_t)(size_t)((lds_void_ptr)(tile + 8 * quarter * ROW_CHUNKS));
+#pragma unroll
+    for (int k = 0; k < FP8_GATHER_INSTR; ++k) {
+        if (64 * k + 64 <= FP8_STAGE_CHUNKS || lane < FP8_STAGE_CHUNKS - 64 * k) {
             asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
                          :
-                         : "v"(off), "s"(kv_b), "s"(lds_base)
+                         : "v"(off[k]), "s"(kv_b), "s"(lds_base + 1024u * k)
                          : "memory", "m0");
         }
-    } else {
-        slots[lane] = make_uint4(0u, 0u, 0u, 0u);
-        if (lane < ROW_CHUNKS - 64) slots[64 + lane] = make_uint4(0u, 0u, 0u, 0u);
     }
 }
 
@@ -582,37 +587,56 @@ __device__ __forceinline__ uint32_t dequant_pair(uint32_t codes, bool upper, flo
     return __builtin_bit_cast(uint32_t, r);
 }
 
-// the 8 rows of quarter `quarter`: codes and scales at positions 31..63 -> bf16 latent values at 0..63. Two
-// rows per step: lanes 0-31 take row 2*j, lanes 32-63 row 2*j + 1; a lane converts 16 codes and reads the
-// scale of its block of 128 straight from the row's scale chunk. All reads of the quarter are issued before the
-// first write (a wavefront's LDS operations execute in order, and the quarter belongs to this wavefront alone).
-// A padding row was zero-filled by the gather: codes 0 times scale 0 writes the same zeros again.
-__device__ __forceinline__ void dequant_quarter(uint4* tile, int quarter, int lane) {
-    asm volatile("" : "+v"(lane));  // (as in gather_issue_fp8: no per-row addresses kept across the tile loop)
+// the 8 rows of quarter `quarter` from the gathered form (see above) to the tile's bf16 layout, rows 4..7 first and
+// then rows 0..3: the bf16 form of rows 4..7 (chunks 288..575 of the region) does not reach the gathered form of
+// rows 0..3 (chunks 0..163), and within a step every read is issued before the first write. Codes: lanes 0-31
+// take one row and lanes 32-63 the next; a lane converts 16 codes with the scale of their block of 128, read
+// straight from the row's scale chunk. Rope values: 8 bytes per lane, row lane / 16 of the step.
+__device__ __forceinline__ void dequant_quarter(uint4* tile, const int* s_idx_tile, bool pad, int quarter, int lane) {
+    asm volatile("" : "+v"(lane));  // (as in gather_quarter_fp8)
     const int sub = lane & 31;
     const int x = 2 * sub;  // bf16 chunks 2*sub and 2*sub + 1 of the row
-    uint4* slots0 = tile + (8 * quarter + (lane >> 5)) * ROW_CHUNKS;
-    uint4 c[4];
-    float sc[4];
+    const int hi = lane >> 5;
+    const int piece = lane & 15;
+    uint4* region = tile + 8 * quarter * ROW_CHUNKS;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const uint4* slots = slots0 + 2 * j * ROW_CHUNKS;
-        c[j] = slots[FP8_FIRST_SLOT + sub];
-        sc[j] = reinterpret_cast<const float*>(slots + FP8_FIRST_SLOT + 32)[sub >> 3];
-    }
-    __builtin_amdgcn_sched_barrier(0);
+    for (int step = 1; step >= 0; --step) {
+        const int rope_row = 4 * step + (lane >> 4);
+        uint4 c[2];
+        float sc[2];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        uint4* slots = slots0 + 2 * j * ROW_CHUNKS;
-        const int swz = row_swizzle(8 * quarter + 2 * j + (lane >> 5));
-        slots[(x & ~7) | ((x ^ swz) & 7)] =
-            make_uint4(dequant_pair(c[j].x, false, sc[j]), dequant_pair(c[j].x, true, sc[j]),
-                       dequant_pair(c[j].y, false, sc[j]), dequant_pair(c[j].y, true, sc[j]));
-        slots[(x & ~7) | (((x + 1) ^ swz) & 7)] =
-            make_uint4(dequant_pair(c[j].z, false, sc[j]), dequant_pair(c[j].z, true, sc[j]),
-                       dequant_pair(c[j].w, false, sc[j]), dequant_pair(c[j].w, true, sc[j]));
+        for (int j = 0; j < 2; ++j) {
+            const uint4* src = region + (4 * step + 2 * j + hi) * FP8_ROW_CHUNKS;
+            c[j] = src[sub];
+            sc[j] = reinterpret_cast<const float*>(src + 32)[sub >> 3];
+        }
+        uint2 rope = reinterpret_cast<const uint2*>(region + rope_row * FP8_ROW_CHUNKS + 33)[piece];
+        if (pad) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const uint32_t keep = s_idx_tile[8 * quarter + 4 * step + 2 * j + hi] < 0 ? 0u : ~0u;
+                c[j].x &= keep, c[j].y &= keep, c[j].z &= keep, c[j].w &= keep;
+            }
+            const uint32_t keep = s_idx_tile[8 * quarter + rope_row] < 0 ? 0u : ~0u;
+            rope.x &= keep, rope.y &= keep;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int row = 4 * step + 2 * j + hi;
+            uint4* slots = region + row * ROW_CHUNKS;
+            const int swz = row_swizzle(8 * quarter + row);
+            slots[(x & ~7) | ((x ^ swz) & 7)] =
+                make_uint4(dequant_pair(c[j].x, false, sc[j]), dequant_pair(c[j].x, true, sc[j]),
+                           dequant_pair(c[j].y, false, sc[j]), dequant_pair(c[j].y, true, sc[j]));
+            slots[(x & ~7) | (((x + 1) ^ swz) & 7)] =
+                make_uint4(dequant_pair(c[j].z, false, sc[j]), dequant_pair(c[j].z, true, sc[j]),
+                           dequant_pair(c[j].w, false, sc[j]), dequant_pair(c[j].w, true, sc[j]));
+        }
+        reinterpret_cast<uint2*>(region + rope_row * ROW_CHUNKS + 64 +
+                                 ((piece >> 1) ^ row_swizzle(8 * quarter + rope_row)))[piece & 1] = rope;
+        __builtin_amdgcn_sched_barrier(0);
     }
-    __builtin_amdgcn_sched_barrier(0);
 }
 
 // grid: x = split, y = request, z = group of 128 heads; 512 lanes. FP8: kv is a cache in the 656-byte e4m3 form.
@@ -680,7 +704,7 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
             raw_key[j] = resolve_key(raw_key[j], b, kva, n_kv_rows);
     }
     if (tid == 0) s_first_masked_tile = n_tiles;
-    for (int c = tid; c < GATHER_TAB; c += 512) {
+    for (int c = tid; c < (FP8 ? 0 : GATHER_TAB); c += 512) {  // (the e4m3 gather computes its offsets itself)
         const int row = c / ROW_CHUNKS;  // 0..7; the tile row is 8*quarter + row: for odd quarters the
         const int pos = c - row * ROW_CHUNKS;  // swizzle term has bit 2 flipped (gather_prepare)
         const int chunk = (pos & ~7) | ((pos ^ row_swizzle(row)) & 7);
@@ -709,11 +733,8 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
     // two groups share the work; from tile 2 on the lag group gathers alone).
     if (group < n_tiles) {
         if constexpr (FP8) {
-            const int keys = s_idx[group * TILE_ROWS + 8 * (wave & 3) + (lane & 7)];  // one LDS read for the 8 rows
-#pragma unroll
-            for (int i = 0; i < FP8_GATHER_INSTR; ++i) {
-                gather_issue_fp8(tiles + group * TILE_CHUNKS, kv_b, __builtin_amdgcn_readlane(keys, i), i, wave & 3, lane);
-            }
+            gather_quarter_fp8(tiles + group * TILE_CHUNKS, kv_b, s_idx + group * TILE_ROWS, group >= first_masked_tile,
+                               wave & 3, lane);
         } else {
             uint32_t off[GATHER_INSTR];
             const bool pad = group >= first_masked_tile;
@@ -788,7 +809,7 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
                 // its rows into bf16 before the barrier below hands the tile to everyone
                 asm volatile("" ::: "memory");  // the reads below stay behind the wait above
                 if (group == (t == 0 ? 0 : 1))
-                    dequant_quarter(tiles + (t % 3) * TILE_CHUNKS, wave & 3, lane);
+                    dequant_quarter(tiles + (t % 3) * TILE_CHUNKS, s_idx + t * TILE_ROWS, t >= first_masked_tile, wave & 3, lane);
             }
         }
         __builtin_amdgcn_s_waitcnt((63 & 15) | ((63 >> 4) << 14) | (7 << 4) | (0 << 8));  // lgkmcnt(0)
@@ -815,11 +836,7 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
             // they go out back to back and the QK^T loop stays free of them.
             if (gather) {
                 if constexpr (FP8) {
-                    const int keys = s_idx[t2 * TILE_ROWS + 8 * (wave & 3) + (lane & 7)];
-#pragma unroll
-                    for (int i = 0; i < FP8_GATHER_INSTR; ++i) {
-                        gather_issue_fp8(gather_tile, kv_b, __builtin_amdgcn_readlane(keys, i), i, wave & 3, lane);
-                    }
+                    gather_quarter_fp8(gather_tile, kv_b, s_idx + t2 * TILE_ROWS, gather_pad, wave & 3, lane);
                 } else {
                     uint32_t goff[GATHER_INSTR];
                     gather_prepare(goff, s_idx + t2 * TILE_ROWS, s_gather_tab, gather_pad, wave & 3, lane);
