@@ -798,18 +798,22 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
         if ((h & 1) == 0 && h < 2 * n_tiles) {
             // tile h/2 must be resident: everything but this wavefront's share of the next tile
             const int t = h >> 1;
-            const bool plain_wait = t + 1 < n_tiles && t + 1 < first_masked_tile && !(FP8 && h == 0);
-            if (plain_wait) {
-                wait_vmcnt<FP8 ? FP8_GATHER_INSTR : GATHER_INSTR>();  // (the lead group has no loads in flight)
-            } else {
-                wait_all_memory();
-            }
             if constexpr (FP8) {
-                // the wavefronts that gathered tile t (the lead group for tile 0, the lag group otherwise) turn
-                // its rows into bf16 before the barrier below hands the tile to everyone
-                asm volatile("" ::: "memory");  // the reads below stay behind the wait above
-                if (group == (t == 0 ? 0 : 1))
-                    dequant_quarter(tiles + (t % 3) * TILE_CHUNKS, s_idx + t * TILE_ROWS, t >= first_masked_tile, wave & 3, lane);
+                // tile 0 was gathered by the lead group: it turns its rows into bf16 here, before the barrier
+                // below hands the tile to everyone; every later tile is converted by the lag group inside the
+                // half-step before (see there)
+                if (h == 0 && group == 0) {
+                    wait_all_memory();
+                    asm volatile("" ::: "memory");  // the reads below stay behind the wait above
+                    dequant_quarter(tiles, s_idx, 0 >= first_masked_tile, wave & 3, lane);
+                }
+            } else {
+                const bool plain_wait = t + 1 < n_tiles && t + 1 < first_masked_tile;
+                if (plain_wait) {
+                    wait_vmcnt<GATHER_INSTR>();  // (the lead group has no loads in flight)
+                } else {
+                    wait_all_memory();
+                }
             }
         }
         __builtin_amdgcn_s_waitcnt((63 & 15) | ((63 >> 4) << 14) | (7 << 4) | (0 << 8));  // lgkmcnt(0)
@@ -861,6 +865,21 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
 #pragma unroll
             for (int qd = 0; qd < 4; ++qd) {
                 my_xchg[qd * 64 + lane] = floatx4{s[4 * qd], s[4 * qd + 1], s[4 * qd + 2], s[4 * qd + 3]};
+            }
+            __builtin_amdgcn_sched_barrier(0);  // (the scores leave their registers before the conversion needs them)
+            if constexpr (FP8) {
+                // the lag group gathered tile t + 1 two half-steps ago: its rows become bf16 here, next to the lead
+                // group's softmax and P V of tile t, and the next barrier hands the tile to everyone
+                if (group == 1 && t + 1 < n_tiles) {
+                    if (gather) {
+                        wait_vmcnt<FP8_GATHER_INSTR>();  // all but the loads of tile t + 2 issued above
+                    } else {
+                        wait_all_memory();
+                    }
+                    asm volatile("" ::: "memory");  // the reads below stay behind the wait above
+                    dequant_quarter(tiles + ((t + 1) % 3) * TILE_CHUNKS, s_idx + (t + 1) * TILE_ROWS,
+                                    t + 1 >= first_masked_tile, wave & 3, lane);
+                }
             }
             PHASE_MARK(3);  // QK^T
         }
