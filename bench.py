@@ -38,7 +38,7 @@ METRIC = "GB/s & % HBM peak (GDN/MoE/MLA decode); fp8 TFLOP/s % MFMA peak (MoE p
 # both in KiB); the counter summary is profiles/all_workloads_hbm_traffic_pmc.md.
 # None = not measured.
 MEASURED_TRAFFIC = {'gdn': 1085972770, 'moe_decode': 6664643628, 'mla': 223326108, 'index_scores': 553871480,
-                    'index_scores_fp8': 289779791, 'moe_prefill': 11230161000}
+                    'index_scores_fp8': 289779791, 'moe_prefill': 11230161000, 'mla_fp8_cache': 172870467}
 
 
 SETTLE_SECONDS = 0.05
@@ -495,7 +495,7 @@ def bench_mla_fp8_cache(torch, capi, dev, steps, warmup, cpu_baseline):
         value=work / sec / 1e9, unit="GB/s", ms_per_step=sec * 1e3, ms_per_step_two_step_form=two_step * 1e3,
         dtype="bf16", kernel="sparse_mla_split8_kernel",
         roofline=dict(bound="hbm", achieved=work / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
-                      frac=work / sec / 1e9 / HBM_PEAK_GBS, traffic=None),
+                      frac=work / sec / 1e9 / HBM_PEAK_GBS, traffic=MEASURED_TRAFFIC['mla_fp8_cache']),
         algorithmic_bytes=work)
 
 
