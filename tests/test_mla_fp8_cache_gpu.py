@@ -50,7 +50,8 @@ def run_bf16(capi, dev, q, kv, idx, dtype=torch.bfloat16, config=0):
 
 
 @pytest.mark.parametrize('shape', [(2, 128, 512, 64), (3, 128, 4096, 2048), (1, 64, 300, 77), (2, 32, 1024, 256),
-                                   (1, 256, 2048, 1024)])
+                                   (1, 256, 2048, 1024), (2, 128, 700, 77), (1, 128, 40, 33), (2, 128, 9, 9),
+                                   (1, 128, 5000, 1000)])
 def test_decode_over_the_fp8_cache(capi, dev, shape):
     B, H, N, topk = shape
     gen = torch.Generator().manual_seed(sum(shape))
