@@ -233,3 +233,40 @@ def test_fp8_indexer_chain_in_a_graph(capi, dev):
         torch.testing.assert_close(sc_g.cpu()[live], want[live], rtol=2e-3, atol=2e-3)
         assert torch.equal(idx_g.cpu(), mla.topk_select(sc_g.cpu(), k, lengths.cpu()))
         eager_noise(dev)
+
+
+def test_fp8_latent_cache_step_in_a_graph(capi, dev):
+    # the new token's latent row is quantised into the e4m3 latent cache, then attended over that cache (the split
+    # kernel dequantises its tiles in LDS: nothing is allocated, cleared or carried over between launches)
+    gen = torch.Generator().manual_seed(23)
+    B, H, N, k = 2, 128, 1024, 256
+    q, kv, idx = mla.mla_make_inputs(B, H, N, k, generator=gen)
+    idx[:, 0] = 9                                            # the row the step writes is always selected
+    idx[1, 4] = -1
+    q, kv, idx = q.to(dev), kv.to(dev), idx.to(dev)
+    cache = torch.empty(B, N, capi.LATENT_ROW_BYTES, dtype=torch.uint8, device=dev)
+    capi.mla_latent_quant_launch(cache, kv)
+    new_row = torch.empty(B, 1, 576, dtype=torch.bfloat16, device=dev)
+    new_bytes = torch.empty(B, 1, capi.LATENT_ROW_BYTES, dtype=torch.uint8, device=dev)
+    ws = torch.empty(capi.sparse_mla_fp8_workspace_bytes(B, H, k), dtype=torch.uint8, device=dev)
+
+    def step(out, ws):
+        capi.mla_latent_quant_launch(new_bytes, new_row)
+        cache[:, 9].copy_(new_bytes[:, 0])
+        capi.sparse_mla_decode_fp8_launch(out, q, cache, idx, ws)
+
+    out_g, out_e = (torch.empty(B, H, 512, device=dev) for _ in range(2))
+    new_row.copy_(torch.randn(B, 1, 576, device=dev))
+    graph = capture(lambda: step(out_g, ws))
+    ws_e = torch.empty_like(ws)
+    for r in range(3):
+        new_row.copy_(torch.randn(B, 1, 576, device=dev) * (r + 1))
+        out_g.fill_(float('nan'))
+        graph.replay()
+        torch.cuda.synchronize()
+        step(out_e, ws_e)
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, out_e)
+        want = mla.sparse_mla_decode_fp8(q.cpu(), cache.cpu(), idx.cpu(), out_dtype=torch.float32)
+        assert mla.rel_rms_error(out_g.cpu(), want) <= 2e-2
+        eager_noise(dev)
