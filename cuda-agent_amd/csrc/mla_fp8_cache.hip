@@ -10,13 +10,15 @@
 //   mla_latent_quant_launcher        bf16 rows [rows, 576] -> rows of 656 bytes (the cache write side)
 //   sparse_mla_decode_fp8_launcher   decode over such a cache
 //
-// Decode runs in two steps. A first kernel gathers the selected rows of every request and dequantises
-// them to bf16 (code * scale in fp32, rounded to nearest even) into a compact per-request block
-// [batch, topk, 576] in the workspace, with an index list 0..topk-1 beside it (-1 where the caller's
-// entry was padding); the decode kernel of sparse_mla.hip then runs on that block unchanged, so the result
-// is bit for bit what sparse_mla_decode_launcher gives on the dequantised cache. The selected rows cross
-// HBM once as 656 bytes; the compact block is written and read back (it is what the step costs over the
-// bf16 cache: the form buys cache capacity, not time).
+// Decode has two forms with the same result, bit for bit what sparse_mla_decode_launcher gives on the
+// dequantised cache (code * scale in fp32, rounded to nearest-even bf16).
+//   * Head counts that are multiples of 128: the 8-wavefront kernel of sparse_mla.hip gathers the 656-byte
+//     rows itself and converts every key tile in LDS (its FP8 instantiation); the selected rows cross HBM once
+//     and nothing else is written.
+//   * Otherwise, or with 5000 added to config, two steps: the kernel below gathers the selected rows of every
+//     request and dequantises them into a compact per-request block [batch, topk, 576] in the workspace, with
+//     an index list 0..topk-1 beside it (-1 where the caller's entry was padding); the decode kernels of
+//     sparse_mla.hip then run on that block unchanged. The compact block is written and read back.
 #include <hip/hip_runtime.h>
 #include <hip/hip_bf16.h>
 #include <stdint.h>
