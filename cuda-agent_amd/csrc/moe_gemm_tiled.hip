@@ -224,7 +224,12 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
 
     const uint32_t stage_base = (uint32_t)(size_t)((lds_void_ptr)s_stage);
     // load i (0..7) of this wavefront's share of stage kb: 0..3 weights, 4..7 activations
-    auto issue_load = [&](int kb, int i, int slot_parity) {
+    // Tiles of at most 128 pairs (the last tile of most experts holds a few dozen) use only the first half of a
+    // stage's activation rows and pair scales. Their K loop is bound by load latency, not by the matrix pipe, so
+    // they request activations and scales two blocks ahead like the weights: block kb's go to stage kb % 2, half
+    // (kb / 2) % 2 (`sub`), and the wavefronts of the first pair half read them there.
+    const bool half_tile = cnt <= TILE_PAIRS / 2;
+    auto issue_load = [&](int kb, int i, int slot_parity, int sub = 0) {
         const uint32_t st = stage_base + (slot_parity & 1) * STAGE_BYTES;
         if (i < 4) {
             dma16(a_src[i] + (size_t)kb * GROUP, (i & 1) ? ld_off_odd : ld_off_even, st + (4 * wave + i) * 1024);
@@ -232,13 +237,21 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
             // (8-row groups past the tile's last pair are not fetched: their LDS rows feed output
             // columns that are never stored. A third of the prefill workload's tile rows is such
             // padding; leaving it out lowers the L2 traffic, the kernel time did not change.)
-            dma16(a_q + (size_t)kb * GROUP, b_off[i - 4], st + STAGE_A + (4 * wave + i - 4) * 1024);
+            dma16(a_q + (size_t)kb * GROUP, b_off[i - 4], st + STAGE_A + sub * (STAGE_B / 2) + (4 * wave + i - 4) * 1024);
         }
     };
-    auto issue_scales = [&](int kb, int slot_parity) {
+    auto issue_scales = [&](int kb, int slot_parity, bool half = false, int sub = 0) {
         const uint32_t st = stage_base + (slot_parity & 1) * STAGE_BYTES;
-        if (wave == 0) dma16(s_src + (size_t)kb * scale_stride, lane * 16, st + STAGE_A + STAGE_B);
+        if (wave == 0) {
+            if (!half) dma16(s_src + (size_t)kb * scale_stride, lane * 16, st + STAGE_A + STAGE_B);
+            else if (lane < 32) dma16(s_src + (size_t)kb * scale_stride, lane * 16, st + STAGE_A + STAGE_B + sub * (STAGE_S / 2));
+        }
     };
+    // loads of one block that a half tile's wavefront may leave in flight at the top of the block before:
+    // its weights (4), its activation row groups and, in wavefront 0, its pair scales
+    int half_tile_in_flight = 4 + (wave == 0 ? 1 : 0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) half_tile_in_flight += (4 * wave + i) * 8 < cnt ? 1 : 0;
 
     // ---- read side -------------------------------------------------------------------------
     // operand of k-step s, 16-byte piece j: chunk 4s + 2*half + j of row r32 (+32*tile)
@@ -273,20 +286,22 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
     //    VALU work hides behind the matrix pipeline with two partial accumulators only.
     // kb1, kb2: kb+1 and kb+2, or 0 past the end (harmless loads that keep the body branch-free;
     // the epilogue waits for them before it reuses the stages).
-    auto block = [&](auto nb_tag, int kb, int kb1, int kb2) {
+    auto block = [&](auto nb_tag, auto half_tag, int kb, int kb1, int kb2) {
         constexpr int NB = decltype(nb_tag)::value;
+        constexpr bool HALF = decltype(half_tag)::value != 0;  // a half tile (compile time: full tiles keep their code)
         const lds_bytes st = stage_ptr + (kb & 1) * STAGE_BYTES;
         intx8 A[2][2];  // [tile][k-step]
         intx8 B[2];     // [k-step]
         float bs = 0.f;
+        const int rh = HALF ? (kb >> 1) & 1 : th;  // half of the stage's pair rows this wavefront reads
         auto read_b = [&](int b) {
-            const lds_bytes bt = st + STAGE_A + (th * 128 + b * 32) * GROUP;
+            const lds_bytes bt = st + STAGE_A + (rh * 128 + b * 32) * GROUP;
             B[0] = join(*(lds_x4)(bt + rd), *(lds_x4)(bt + (rd ^ 16)));
             B[1] = join(*(lds_x4)(bt + (rd ^ 64)), *(lds_x4)(bt + (rd ^ 64 ^ 16)));
         };
         auto read_bs = [&](int b) {
             return *(const __attribute__((address_space(3))) float*)(st + STAGE_A + STAGE_B +
-                                                                     (th * 128 + b * 32 + r32) * 4);
+                                                                     (rh * 128 + b * 32 + r32) * 4);
         };
         if (NB > 0) {
 #pragma unroll
@@ -307,9 +322,15 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
         // load sequence of the block: pair scales and activations of block kb+1 (load numbers
         // 0..3), then the weights of block kb+2 (4..7), spread over the MFMA pairs
         auto load_number = [&](int n) {
-            if (n == 0) issue_scales(kb1, kb + 1);
-            if (n < 4) issue_load(kb1, 4 + n, kb + 1);
-            else issue_load(kb2, n - 4, kb);
+            if constexpr (HALF) {
+                if (n == 0) issue_scales(kb2, kb, true, ((kb + 2) >> 1) & 1);
+                if (n < 4) issue_load(kb2, 4 + n, kb, ((kb + 2) >> 1) & 1);
+                else issue_load(kb2, n - 4, kb);
+            } else {
+                if (n == 0) issue_scales(kb1, kb + 1);
+                if (n < 4) issue_load(kb1, 4 + n, kb + 1);
+                else issue_load(kb2, n - 4, kb);
+            }
         };
         constexpr int PER_SLOT = NB >= 3 ? 2 : NB == 2 ? 2 : NB == 1 ? 4 : 8;
         auto loads = [&](int slot) {
@@ -377,22 +398,40 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
     };
 
     PHASE_TIMING_BEGIN();
-    issue_scales(0, 0);
+    issue_scales(0, 0, half_tile, 0);
 #pragma unroll
     for (int i = 4; i < 8; ++i) issue_load(0, i, 0);
 #pragma unroll
     for (int i = 0; i < 4; ++i) issue_load(0, i, 0);
     if (KB > 1) {
+        if (half_tile) {
+            issue_scales(1, 1, true, 0);
+#pragma unroll
+            for (int i = 4; i < 8; ++i) issue_load(1, i, 1);
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i) issue_load(1, i, 1);
     }
     PHASE_MARK(0);  // prologue
     // the K loop exists once per value of NB, so that the accumulators live in one place per copy
-    auto k_loop = [&](auto nb_tag) {
+    auto k_loop = [&](auto nb_tag, auto half_tag) {
+        constexpr bool HALF = decltype(half_tag)::value != 0;
         for (int kb = 0; kb < KB; ++kb) {
             if (KB > 1) {
-                // everything but the 4 weight loads of block kb+1 (past the end: harmless ones)
-                __builtin_amdgcn_s_waitcnt((4 & 15) | ((4 >> 4) << 14) | (7 << 4) | (15 << 8));
+                // everything but the 4 weight loads of block kb+1 (past the end: harmless ones); in a half tile
+                // everything but the loads of block kb+1
+                if constexpr (!HALF) {
+                    __builtin_amdgcn_s_waitcnt((4 & 15) | ((4 >> 4) << 14) | (7 << 4) | (15 << 8));
+                } else {
+                    switch (half_tile_in_flight) {
+                        case 4: __builtin_amdgcn_s_waitcnt(4 | (7 << 4) | (15 << 8)); break;
+                        case 5: __builtin_amdgcn_s_waitcnt(5 | (7 << 4) | (15 << 8)); break;
+                        case 6: __builtin_amdgcn_s_waitcnt(6 | (7 << 4) | (15 << 8)); break;
+                        case 7: __builtin_amdgcn_s_waitcnt(7 | (7 << 4) | (15 << 8)); break;
+                        case 8: __builtin_amdgcn_s_waitcnt(8 | (7 << 4) | (15 << 8)); break;
+                        default: __builtin_amdgcn_s_waitcnt(9 | (7 << 4) | (15 << 8)); break;
+                    }
+                }
                 asm volatile("" ::: "memory");
             } else {
                 wait_all_loads();
@@ -401,17 +440,27 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
             PHASE_MARK(2);  // wait for the other wavefronts
-            block(nb_tag, kb, kb + 1 < KB ? kb + 1 : 0, kb + 2 < KB ? kb + 2 : 0);
+            block(nb_tag, half_tag, kb, kb + 1 < KB ? kb + 1 : 0, kb + 2 < KB ? kb + 2 : 0);
             asm volatile("" ::: "memory");
             PHASE_MARK(4);  // operand reads, MFMAs, promotion, loads of later blocks
         }
     };
-    switch (active_b) {
-        case 4: k_loop(IntConstant<4>{}); break;
-        case 3: k_loop(IntConstant<3>{}); break;
-        case 2: k_loop(IntConstant<2>{}); break;
-        case 1: k_loop(IntConstant<1>{}); break;
-        default: k_loop(IntConstant<0>{}); break;
+    if (!half_tile) {
+        switch (active_b) {
+            case 4: k_loop(IntConstant<4>{}, IntConstant<0>{}); break;
+            case 3: k_loop(IntConstant<3>{}, IntConstant<0>{}); break;
+            case 2: k_loop(IntConstant<2>{}, IntConstant<0>{}); break;
+            case 1: k_loop(IntConstant<1>{}, IntConstant<0>{}); break;
+            default: k_loop(IntConstant<0>{}, IntConstant<0>{}); break;
+        }
+    } else {
+        switch (active_b) {
+            case 4: k_loop(IntConstant<4>{}, IntConstant<1>{}); break;
+            case 3: k_loop(IntConstant<3>{}, IntConstant<1>{}); break;
+            case 2: k_loop(IntConstant<2>{}, IntConstant<1>{}); break;
+            case 1: k_loop(IntConstant<1>{}, IntConstant<1>{}); break;
+            default: k_loop(IntConstant<0>{}, IntConstant<1>{}); break;
+        }
     }
     wait_all_loads();
     __syncthreads();  // the stages are free: reuse them for the epilogue exchange
