@@ -1281,7 +1281,8 @@ extern "C" void sparse_mla_decode_paged_launcher(void* out, const void* q, const
 }
 
 // Decode over a cache in the 656-byte e4m3 form with the dequantisation inside the 128-head kernel (see
-// gather_issue_fp8 / dequant_quarter). Returns 1 if the launch was made (or rejected with a status), 0 if
+// gather_quarter_fp8 / dequant_quarter). Internal to the library: mla_fp8_cache.hip calls it from
+// sparse_mla_decode_fp8_launcher and its paged form; it is not part of the public header. Returns 1 if the launch was made (or rejected with a status), 0 if
 // this shape has to take the two-step form of sparse_mla_decode_fp8_launcher: head counts other than
 // multiples of 128, config >= 1000, caches of 4 GB and more per addressed block.
 // block_table / table_stride / page_shift / batch_rows: the addressing of the cache, as in KvAddressing.
