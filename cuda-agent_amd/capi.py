@@ -496,7 +496,7 @@ def topk_select_launch(idx_out, scores, lengths=None, stream=None):
 
 
 MOE_WORKSPACE_FIELDS = ('ids', 'weights', 'expert_offsets', 'sorted_pairs', 'pair_pos', 'x_q', 'x_s',
-                        'h_q', 'h_s', 'y')
+                        'h_q', 'h_s', 'y', 'h_marks')
 
 
 def moe_workspace_bytes(tokens, hidden, inter, n_experts, top_k=8):
@@ -506,7 +506,7 @@ def moe_workspace_bytes(tokens, hidden, inter, n_experts, top_k=8):
 def moe_workspace_views(workspace, tokens, hidden, inter, n_experts, top_k=8):
     """Typed views of the intermediate buffers inside a workspace tensor (uint8, 1-D)."""
     import torch
-    offs = (c_size_t * 10)()
+    offs = (c_size_t * len(MOE_WORKSPACE_FIELDS))()
     library().moe_fp8_workspace_layout(offs, tokens, hidden, inter, n_experts, top_k)
     pairs = tokens * top_k
     spec = {
@@ -515,6 +515,7 @@ def moe_workspace_views(workspace, tokens, hidden, inter, n_experts, top_k=8):
         'pair_pos': (torch.int32, (pairs,)), 'x_q': (torch.float8_e4m3fn, (tokens, hidden)),
         'x_s': (torch.float32, (tokens, hidden // 128)), 'h_q': (torch.float8_e4m3fn, (pairs, inter)),
         'h_s': (torch.float32, (pairs, inter // 128)), 'y': (torch.float32, (pairs, hidden)),
+        'h_marks': (torch.uint8, (pairs, inter)),
     }
     views = {}
     for name, off in zip(MOE_WORKSPACE_FIELDS, offs):

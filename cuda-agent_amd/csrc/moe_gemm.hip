@@ -38,9 +38,95 @@ __device__ __forceinline__ intx8 join(intx4 lo, intx4 hi) {
 
 __device__ __forceinline__ float silu(float x) { return x / (1.f + expf(-x)); }
 
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// 8 e4m3 codes (two dwords) -> 8 bf16, exactly (every e4m3 value is a bf16 value)
+__device__ __forceinline__ bf16x8 e4m3x8_to_bf16(int lo, int hi) {
+    const bf16x2 a = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, false);
+    const bf16x2 b = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, true);
+    const bf16x2 c = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, false);
+    const bf16x2 d = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, true);
+    return bf16x8{a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
+}
+
+// A lane's 32 operand bytes of one 128-block as the operands of four v_mfma_f32_16x16x32_bf16 steps:
+// step s takes bytes 8s..8s+7 of the lane (which 32 of the block's 128 elements a step covers is
+// immaterial as long as both operands are cut the same way).
+struct Bf16Block {
+    bf16x8 step[4];
+};
+__device__ __forceinline__ Bf16Block to_bf16_block(intx8 v) {
+    Bf16Block r;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) r.step[s] = e4m3x8_to_bf16(v[2 * s], v[2 * s + 1]);
+    return r;
+}
+
+// Unscaled dot products of one 128-block for 16 weight rows x 16 pairs.
+// EXACT: on the bf16 matrix core, which adds the (exact) products without losing bits that matter (measured
+// on gfx950: |error| <= 2^-25 of the sum of |products|, against 2^-16 for the e4m3 instruction), so that the
+// requantised codes of h agree with an fp32 evaluation. Otherwise one e4m3 instruction.
+__device__ __forceinline__ floatx4 block_dot_bf16(const Bf16Block& a, const Bf16Block& b) {
+    floatx4 part = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < 4; ++s) part = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.step[s], b.step[s], part, 0, 0, 0);
+    return part;
+}
+
+// Epilogue of the streaming gate/up kernels: h = silu(gate) * up, e4m3 with one scale per pair over the
+// workgroup's 128 columns. acc[nt][t]: tiles 0, 1 gate, 2, 3 up; a lane holds rows 4g..4g+3 of each 16-row
+// tile for pair column `col`.
+template <int NT>
+__device__ __forceinline__ void gate_up_epilogue(const floatx4 (&acc)[NT][4], float (*s_amax)[NT * 16],
+                                                 const int (&pos)[NT], int end, uint8_t* __restrict__ h_q,
+                                                 float* __restrict__ h_s, int inter, int rb, int wave, int col,
+                                                 int g, bool pow2) {
+    floatx4 h[NT][2];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        float amax = 0.f;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float v = silu(acc[nt][i][r]) * acc[nt][2 + i][r];
+                h[nt][i][r] = v;
+                amax = fmaxf(amax, fabsf(v));
+            }
+        }
+        amax = fmaxf(amax, __shfl_xor(amax, 16));
+        amax = fmaxf(amax, __shfl_xor(amax, 32));
+        if (g == 0) s_amax[wave][nt * 16 + col] = amax;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int idx = nt * 16 + col;
+        const float amax =
+            fmaxf(fmaxf(s_amax[0][idx], s_amax[1][idx]), fmaxf(s_amax[2][idx], s_amax[3][idx]));
+        const float scale = group_scale(amax, pow2);
+        if (pos[nt] < end) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                float q[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    q[r] = fminf(fmaxf(h[nt][i][r] / scale, -E4M3_MAX), E4M3_MAX);
+                }
+                int packed = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], 0, false);
+                packed = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], packed, true);
+                *reinterpret_cast<int*>(h_q + (size_t)pos[nt] * inter + rb * GROUP + wave * 32 + i * 16 +
+                                        4 * g) = packed;
+            }
+            if (wave == 0 && g == 0) h_s[(size_t)pos[nt] * (inter / GROUP) + rb] = scale;
+        }
+    }
+}
+
 // GATE_UP: 4 weight tiles per wavefront (2 gate + 2 up), output h_q/h_s.
 // otherwise: 2 weight tiles per wavefront, output y.
-template <bool GATE_UP, int NT>
+template <bool GATE_UP, int NT, bool EXACT = false>
 __global__ __launch_bounds__(256) void moe_stream_gemm_kernel(
     const uint8_t* __restrict__ w_q, const float* __restrict__ w_s, const uint8_t* __restrict__ a_q,
     const float* __restrict__ a_s, const int* __restrict__ sorted_pairs,
@@ -117,6 +203,21 @@ __global__ __launch_bounds__(256) void moe_stream_gemm_kernel(
             if (GATE_UP) w_scale[buf][1] = ws_ptr[1][kb];
         };
         auto compute_block = [&](int buf) {
+            if constexpr (EXACT) {
+                Bf16Block a[TILES];
+#pragma unroll
+                for (int t = 0; t < TILES; ++t) a[t] = to_bf16_block(join(a_lo[buf][t], a_hi[buf][t]));
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const Bf16Block b = to_bf16_block(join(b_lo[buf][nt], b_hi[buf][nt]));
+#pragma unroll
+                    for (int t = 0; t < TILES; ++t) {
+                        const float s = b_scale[buf][nt] * w_scale[buf][GATE_UP ? (t >> 1) : 0];
+                        acc[nt][t] += block_dot_bf16(a[t], b) * s;
+                    }
+                }
+                return;
+            }
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 const intx8 b = join(b_lo[buf][nt], b_hi[buf][nt]);
@@ -141,48 +242,8 @@ __global__ __launch_bounds__(256) void moe_stream_gemm_kernel(
             }
         }
 
-        if (GATE_UP) {
-            // h = silu(gate) * up, then e4m3 with one scale per pair over this block's 128 columns
-            floatx4 h[NT][2];
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                float amax = 0.f;
-#pragma unroll
-                for (int i = 0; i < 2; ++i) {
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const float v = silu(acc[nt][i][r]) * acc[nt][2 + i][r];
-                        h[nt][i][r] = v;
-                        amax = fmaxf(amax, fabsf(v));
-                    }
-                }
-                amax = fmaxf(amax, __shfl_xor(amax, 16));
-                amax = fmaxf(amax, __shfl_xor(amax, 32));
-                if (g == 0) s_amax[wave][nt * 16 + col] = amax;
-            }
-            __syncthreads();
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                const int idx = nt * 16 + col;
-                const float amax =
-                    fmaxf(fmaxf(s_amax[0][idx], s_amax[1][idx]), fmaxf(s_amax[2][idx], s_amax[3][idx]));
-                const float scale = group_scale(amax, pow2);
-                if (pos[nt] < end) {
-#pragma unroll
-                    for (int i = 0; i < 2; ++i) {
-                        float q[4];
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) {
-                            q[r] = fminf(fmaxf(h[nt][i][r] / scale, -E4M3_MAX), E4M3_MAX);
-                        }
-                        int packed = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], 0, false);
-                        packed = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], packed, true);
-                        *reinterpret_cast<int*>(h_q + (size_t)pos[nt] * inter + rb * GROUP + wave * 32 +
-                                                i * 16 + 4 * g) = packed;
-                    }
-                    if (wave == 0 && g == 0) h_s[(size_t)pos[nt] * (inter / GROUP) + rb] = scale;
-                }
-            }
+        if constexpr (GATE_UP) {
+            gate_up_epilogue<NT>(acc, s_amax, pos, end, h_q, h_s, inter, rb, wave, col, g, pow2);
             __syncthreads();  // s_amax is reused by the next pass
         } else {
 #pragma unroll
@@ -241,7 +302,7 @@ __device__ __forceinline__ void dma16_ptr(const void* lane_ptr, uint32_t lds_bas
                  : "memory", "m0");
 }
 
-template <bool GATE_UP, int NT>
+template <bool GATE_UP, int NT, bool EXACT = false>
 __global__ __launch_bounds__(256) void moe_stream_gemm_lds_kernel(
     const uint8_t* __restrict__ w_q, const float* __restrict__ w_s, const uint8_t* __restrict__ a_q,
     const float* __restrict__ a_s, const int* __restrict__ sorted_pairs,
@@ -379,63 +440,41 @@ __global__ __launch_bounds__(256) void moe_stream_gemm_lds_kernel(
                 const intx4 hi = *(lds_x4)(stage + t * TILE_BYTES + (rd_off ^ 64));
                 a[t] = join(lo, hi);
             }
+            if constexpr (EXACT) {
+                Bf16Block ab[TILES];
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                const intx4 lo = *(lds_x4)(stage + (TILES + nt) * TILE_BYTES + rd_off);
-                const intx4 hi = *(lds_x4)(stage + (TILES + nt) * TILE_BYTES + (rd_off ^ 64));
-                const intx8 b = join(lo, hi);
-                const float bs = s_bscale[kb][nt * 16 + col];
+                for (int t = 0; t < TILES; ++t) ab[t] = to_bf16_block(a[t]);
 #pragma unroll
-                for (int t = 0; t < TILES; ++t) {
-                    const floatx4 part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                        a[t], b, floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
-                    acc[nt][t] += part * (bs * ((t >> 1) ? ws1 : ws0));
+                for (int nt = 0; nt < NT; ++nt) {
+                    const intx4 lo = *(lds_x4)(stage + (TILES + nt) * TILE_BYTES + rd_off);
+                    const intx4 hi = *(lds_x4)(stage + (TILES + nt) * TILE_BYTES + (rd_off ^ 64));
+                    const Bf16Block b = to_bf16_block(join(lo, hi));
+                    const float bs = s_bscale[kb][nt * 16 + col];
+#pragma unroll
+                    for (int t = 0; t < TILES; ++t) {
+                        acc[nt][t] += block_dot_bf16(ab[t], b) * (bs * ((t >> 1) ? ws1 : ws0));
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const intx4 lo = *(lds_x4)(stage + (TILES + nt) * TILE_BYTES + rd_off);
+                    const intx4 hi = *(lds_x4)(stage + (TILES + nt) * TILE_BYTES + (rd_off ^ 64));
+                    const intx8 b = join(lo, hi);
+                    const float bs = s_bscale[kb][nt * 16 + col];
+#pragma unroll
+                    for (int t = 0; t < TILES; ++t) {
+                        const floatx4 part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                            a[t], b, floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+                        acc[nt][t] += part * (bs * ((t >> 1) ? ws1 : ws0));
+                    }
                 }
             }
             asm volatile("" ::: "memory");  // this stage's LDS reads stay above the next refill
         }
 
-        if (GATE_UP) {
-            floatx4 h[NT][2];
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                float amax = 0.f;
-#pragma unroll
-                for (int i = 0; i < 2; ++i) {
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const float v = silu(acc[nt][i][r]) * acc[nt][2 + i][r];
-                        h[nt][i][r] = v;
-                        amax = fmaxf(amax, fabsf(v));
-                    }
-                }
-                amax = fmaxf(amax, __shfl_xor(amax, 16));
-                amax = fmaxf(amax, __shfl_xor(amax, 32));
-                if (g == 0) s_amax[wave][nt * 16 + col] = amax;
-            }
-            __syncthreads();
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                const int idx = nt * 16 + col;
-                const float amax =
-                    fmaxf(fmaxf(s_amax[0][idx], s_amax[1][idx]), fmaxf(s_amax[2][idx], s_amax[3][idx]));
-                const float scale = group_scale(amax, pow2);
-                if (pos[nt] < end) {
-#pragma unroll
-                    for (int i = 0; i < 2; ++i) {
-                        float q[4];
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) {
-                            q[r] = fminf(fmaxf(h[nt][i][r] / scale, -E4M3_MAX), E4M3_MAX);
-                        }
-                        int packed = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], 0, false);
-                        packed = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], packed, true);
-                        *reinterpret_cast<int*>(h_q + (size_t)pos[nt] * inter + rb * GROUP + wave * 32 +
-                                                i * 16 + 4 * g) = packed;
-                    }
-                    if (wave == 0 && g == 0) h_s[(size_t)pos[nt] * (inter / GROUP) + rb] = scale;
-                }
-            }
+        if constexpr (GATE_UP) {
+            gate_up_epilogue<NT>(acc, s_amax, pos, end, h_q, h_s, inter, rb, wave, col, g, pow2);
         } else {
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
@@ -463,6 +502,9 @@ bool check_common(int hidden, int inter, int n_experts) {
 // w13_s [E, 2*inter/128, hidden/128].
 // config: 0 sizes the pass from the average pairs per expert; 1, 2, 4 force 16, 32, 64 pairs per
 // pass; adding 8 selects the kernel that loads MFMA operands directly instead of staging in LDS.
+// The block products run on the bf16 matrix core (codes converted in registers; exact sums, so that the
+// requantised h agrees with an fp32 evaluation); +512 (CONFIG_APPROX_REQUANT): on the e4m3 matrix core,
+// whose sums carry about 16 bits.
 extern "C" void moe_gate_up_launcher(void* h_q, float* h_s, const void* x_q, const float* x_s,
                                      const void* w13_q, const float* w13_s, const int* sorted_pairs,
                                      const int* expert_offsets, int tokens, int hidden, int inter,
@@ -484,42 +526,33 @@ extern "C" void moe_gate_up_launcher(void* h_q, float* h_s, const void* x_q, con
     const auto* wq = static_cast<const uint8_t*>(w13_q);
     const bool pow2 = (config & CONFIG_UE8M0) != 0;
     const bool last_first = (config & CONFIG_LAST_EXPERT_FIRST) != 0;
-    config &= ~(CONFIG_UE8M0 | CONFIG_LAST_EXPERT_FIRST);
+    const bool exact = (config & CONFIG_APPROX_REQUANT) == 0;
+    config &= ~(CONFIG_UE8M0 | CONFIG_LAST_EXPERT_FIRST | CONFIG_REQUANT_BITS);
     int nt = config & 7;
     if (nt != 1 && nt != 2 && nt != 4) {
         const long avg = (long)tokens * top_k / n_experts;  // pairs per expert if spread evenly
         nt = avg <= 16 ? 1 : avg <= 32 ? 2 : 4;
     }
-    const bool lds_path = config < 8 && hidden / GROUP <= 64;  // config 8+nt: direct-operand loads
+    const bool lds_path = config < 8 && hidden / GROUP <= 64 && nt < 4;  // config 8+nt: direct-operand loads
+#define MOE_GATE_UP_LAUNCH(KERNEL, NT_, EXACT_)                                                           \
+    KERNEL<true, NT_, EXACT_><<<grid, 256, 0, stream>>>(wq, w13_s, xq, x_s, sorted_pairs, expert_offsets, \
+                                                       hq, h_s, nullptr, hidden, 2 * inter, inter, top_k, \
+                                                       pow2, last_first)
+#define MOE_GATE_UP_CASE(NT_)                                                           \
+    if (lds_path && exact) MOE_GATE_UP_LAUNCH(moe_stream_gemm_lds_kernel, NT_, true);   \
+    else if (lds_path) MOE_GATE_UP_LAUNCH(moe_stream_gemm_lds_kernel, NT_, false);      \
+    else if (exact) MOE_GATE_UP_LAUNCH(moe_stream_gemm_kernel, NT_, true);              \
+    else MOE_GATE_UP_LAUNCH(moe_stream_gemm_kernel, NT_, false)
     switch (nt) {
-        case 1:
-            if (lds_path) {
-                moe_stream_gemm_lds_kernel<true, 1><<<grid, 256, 0, stream>>>(
-                    wq, w13_s, xq, x_s, sorted_pairs, expert_offsets, hq, h_s, nullptr, hidden,
-                    2 * inter, inter, top_k, pow2, last_first);
-            } else {
-                moe_stream_gemm_kernel<true, 1><<<grid, 256, 0, stream>>>(
-                    wq, w13_s, xq, x_s, sorted_pairs, expert_offsets, hq, h_s, nullptr, hidden,
-                    2 * inter, inter, top_k, pow2, last_first);
-            }
-            break;
-        case 2:
-            if (lds_path) {
-                moe_stream_gemm_lds_kernel<true, 2><<<grid, 256, 0, stream>>>(
-                    wq, w13_s, xq, x_s, sorted_pairs, expert_offsets, hq, h_s, nullptr, hidden,
-                    2 * inter, inter, top_k, pow2, last_first);
-            } else {
-                moe_stream_gemm_kernel<true, 2><<<grid, 256, 0, stream>>>(
-                    wq, w13_s, xq, x_s, sorted_pairs, expert_offsets, hq, h_s, nullptr, hidden,
-                    2 * inter, inter, top_k, pow2, last_first);
-            }
-            break;
+        case 1: MOE_GATE_UP_CASE(1); break;
+        case 2: MOE_GATE_UP_CASE(2); break;
         default:
-            moe_stream_gemm_kernel<true, 4><<<grid, 256, 0, stream>>>(
-                wq, w13_s, xq, x_s, sorted_pairs, expert_offsets, hq, h_s, nullptr, hidden, 2 * inter,
-                inter, top_k, pow2, last_first);
+            if (exact) MOE_GATE_UP_LAUNCH(moe_stream_gemm_kernel, 4, true);
+            else MOE_GATE_UP_LAUNCH(moe_stream_gemm_kernel, 4, false);
             break;
     }
+#undef MOE_GATE_UP_CASE
+#undef MOE_GATE_UP_LAUNCH
 }
 
 // y [pairs, hidden] fp32 (rows in sorted order) from h_q/h_s and w2_q [E, hidden, inter] e4m3,
@@ -544,7 +577,7 @@ extern "C" void moe_down_launcher(float* y, const void* h_q, const float* h_s, c
     const auto* wq = static_cast<const uint8_t*>(w2_q);
     const bool last_first = (config & CONFIG_LAST_EXPERT_FIRST) != 0;
     // (the down GEMM has no requantisation: nothing depends on the scale convention)
-    config &= ~(CONFIG_UE8M0 | CONFIG_LAST_EXPERT_FIRST);
+    config &= ~(CONFIG_UE8M0 | CONFIG_LAST_EXPERT_FIRST | CONFIG_REQUANT_BITS);
     int nt = config & 7;
     if (nt != 1 && nt != 2 && nt != 4) {
         const long avg = (long)tokens * top_k / n_experts;

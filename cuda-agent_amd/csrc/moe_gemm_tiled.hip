@@ -147,13 +147,15 @@ __device__ unsigned long long g_phase_cycles[8][8];
 // (v_mfma_scale_f32_32x32x64_f8f6f4: each lane's 32 values of A and of B are multiplied by
 // 2^(byte - 127)), the products of all K blocks add up in the accumulator itself, and the per-block
 // multiply-add on the VALU (128 per wavefront and K block) disappears.
-template <bool GATE_UP, bool UE8M0>
+// FIX (gate/up only): the epilogue also writes the marks of the exact requantisation (moe_common.hpp).
+template <bool GATE_UP, bool UE8M0, bool FIX = false>
 __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
     const uint8_t* __restrict__ w_q, const float* __restrict__ w_s, const uint8_t* __restrict__ a_q,
     const float* __restrict__ as_t, const int* __restrict__ sorted_pairs,
     const int* __restrict__ expert_offsets, const int* __restrict__ tile_start,
     uint8_t* __restrict__ h_q, float* __restrict__ h_s, float* __restrict__ hs_t, float* __restrict__ y,
-    int K, int n_rows, int inter, int top_k, int n_experts, int scale_stride) {
+    int K, int n_rows, int inter, int top_k, int n_experts, int scale_stride,
+    uint8_t* __restrict__ h_marks = nullptr, float err_coef = 0.f) {
     __shared__ __attribute__((aligned(16))) uint8_t s_stage[2 * STAGE_BYTES];
 
     // Workgroup -> (row tile, pair tile). Consecutive workgroup ids go round-robin to the 8 XCDs,
@@ -474,18 +476,38 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
         float* s_amax = reinterpret_cast<float*>(s_stage);                      // [4 row groups][256 pairs]
         constexpr int CODE_ROW = GROUP + 16;                                    // bytes per pair row of codes
         uint8_t* s_codes = s_stage + 4 * TILE_PAIRS * sizeof(float);            // [256 pairs][CODE_ROW]
-        static_assert(4 * TILE_PAIRS * sizeof(float) + TILE_PAIRS * CODE_ROW <= 2 * STAGE_BYTES, "epilogue LDS");
+        // FIX: marks staged like the codes, and three more per-pair statistics
+        uint8_t* s_marks = s_codes + TILE_PAIRS * CODE_ROW;
+        float* s_sumsq = reinterpret_cast<float*>(s_marks + TILE_PAIRS * CODE_ROW);
+        float* s_umax = s_sumsq + 4 * TILE_PAIRS;
+        float* s_sgmax = s_umax + 4 * TILE_PAIRS;
+        static_assert(16 * TILE_PAIRS * sizeof(float) + 2 * TILE_PAIRS * CODE_ROW <= 2 * STAGE_BYTES, "epilogue LDS");
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
-            float m = 0.f;
+            float m = 0.f, sumsq = 0.f, umax = 0.f, sgmax = 0.f;
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                const float v = silu(acc[0][b][i]) * acc[1][b][i];
-                acc[0][b][i] = v;
+                const float sg = silu(acc[0][b][i]);
+                const float v = sg * acc[1][b][i];
+                if constexpr (FIX) {
+                    // (the gate value stays in its register: the second pass needs silu(g) and u again)
+                    sumsq += acc[0][b][i] * acc[0][b][i] + acc[1][b][i] * acc[1][b][i];
+                    umax = fmaxf(umax, fabsf(acc[1][b][i]));
+                    sgmax = fmaxf(sgmax, fabsf(sg));
+                } else {
+                    acc[0][b][i] = v;
+                }
                 m = fmaxf(m, fabsf(v));
             }
             m = fmaxf(m, __shfl_xor(m, 32));
-            if (half == 0) s_amax[rg * TILE_PAIRS + th * 128 + b * 32 + r32] = m;
+            const int at = rg * TILE_PAIRS + th * 128 + b * 32 + r32;
+            if (half == 0) s_amax[at] = m;
+            if constexpr (FIX) {
+                sumsq += __shfl_xor(sumsq, 32);
+                umax = fmaxf(umax, __shfl_xor(umax, 32));
+                sgmax = fmaxf(sgmax, __shfl_xor(sgmax, 32));
+                if (half == 0) s_sumsq[at] = sumsq, s_umax[at] = umax, s_sgmax[at] = sgmax;
+            }
         }
         __syncthreads();
 #pragma unroll
@@ -494,16 +516,40 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
             const float m = fmaxf(fmaxf(s_amax[pl], s_amax[TILE_PAIRS + pl]),
                                   fmaxf(s_amax[2 * TILE_PAIRS + pl], s_amax[3 * TILE_PAIRS + pl]));
             const float scale = group_scale(m, UE8M0);
+            float err = 0.f, dh_max = 0.f;
+            bool uncertain = false;
+            if constexpr (FIX) {
+                const float sumsq = s_sumsq[pl] + s_sumsq[TILE_PAIRS + pl] + s_sumsq[2 * TILE_PAIRS + pl] +
+                                    s_sumsq[3 * TILE_PAIRS + pl];
+                const float umax = fmaxf(fmaxf(s_umax[pl], s_umax[TILE_PAIRS + pl]),
+                                         fmaxf(s_umax[2 * TILE_PAIRS + pl], s_umax[3 * TILE_PAIRS + pl]));
+                const float sgmax = fmaxf(fmaxf(s_sgmax[pl], s_sgmax[TILE_PAIRS + pl]),
+                                          fmaxf(s_sgmax[2 * TILE_PAIRS + pl], s_sgmax[3 * TILE_PAIRS + pl]));
+                err = err_coef * sqrtf(sumsq * (1.f / 256.f));
+                dh_max = (1.1f * umax + sgmax) * err;
+                uncertain = !UE8M0 || group_scale(m + dh_max, true) != group_scale(m - dh_max, true);
+            }
 #pragma unroll
             for (int qd = 0; qd < 4; ++qd) {
                 float q[4];
+                uint32_t marks = 0;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    q[r] = fminf(fmaxf(acc[0][b][4 * qd + r] / scale, -E4M3_MAX), E4M3_MAX);
+                    float v = acc[0][b][4 * qd + r];
+                    if constexpr (FIX) {
+                        const float sg = silu(v);
+                        v = sg * acc[1][b][4 * qd + r];
+                        marks |= requant_marks(v, sg, acc[1][b][4 * qd + r], scale, fmaxf(m, AMAX_FLOOR), err, dh_max,
+                                               uncertain)
+                                 << (8 * r);
+                    }
+                    q[r] = fminf(fmaxf(v / scale, -E4M3_MAX), E4M3_MAX);
                 }
                 int packed = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], 0, false);
                 packed = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], packed, true);
                 *reinterpret_cast<int*>(s_codes + pl * CODE_ROW + rg * 32 + 8 * qd + 4 * half) = packed;
+                if constexpr (FIX)
+                    *reinterpret_cast<uint32_t*>(s_marks + pl * CODE_ROW + rg * 32 + 8 * qd + 4 * half) = marks;
             }
             if (rg == 0 && half == 0 && pl < cnt) {
                 const size_t pos = (size_t)begin + pl;
@@ -517,8 +563,12 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
         for (int it = 0; it < 4; ++it) {
             const int pl = (wave * 4 + it) * 8 + (lane >> 3);
             if (pl < cnt) {
-                const intx4 v = *reinterpret_cast<const intx4*>(s_codes + pl * CODE_ROW + (lane & 7) * 16);
-                *reinterpret_cast<intx4*>(h_q + ((size_t)begin + pl) * inter + rb * GROUP + (lane & 7) * 16) = v;
+                const size_t at = ((size_t)begin + pl) * inter + rb * GROUP + (lane & 7) * 16;
+                *reinterpret_cast<intx4*>(h_q + at) =
+                    *reinterpret_cast<const intx4*>(s_codes + pl * CODE_ROW + (lane & 7) * 16);
+                if constexpr (FIX)
+                    *reinterpret_cast<intx4*>(h_marks + at) =
+                        *reinterpret_cast<const intx4*>(s_marks + pl * CODE_ROW + (lane & 7) * 16);
             }
         }
     } else {
@@ -571,18 +621,25 @@ extern "C" void moe_tiled_prepare_launcher(int* tile_start, float* xs_t, const f
                                            int tokens, int hidden, int n_experts, int top_k,
                                            int scale_stride, hipStream_t stream) {
     if (tokens <= 0) return;
+    if (n_experts <= 0 || n_experts > 1024 || hidden <= 0 || hidden % GROUP != 0 || top_k <= 0) {
+        caa::set_status(CAA_UNSUPPORTED_SHAPE);  // (the tile scan is one workgroup of 1024 lanes)
+        return;
+    }
     const int pairs = tokens * top_k;
     moe_tile_start_kernel<<<1, 1024, 0, stream>>>(expert_offsets, tile_start, n_experts);
     moe_gather_scales_kernel<<<(pairs + 255) / 256, 256, 0, stream>>>(x_s, sorted_pairs, xs_t, pairs,
                                                                     scale_stride, hidden / GROUP, top_k);
 }
 
-extern "C" void moe_gate_up_tiled_launcher(void* h_q, float* h_s, float* hs_t, const void* x_q,
-                                           const float* xs_t, const void* w13_q, const float* w13_s,
-                                           const int* sorted_pairs, const int* expert_offsets,
-                                           const int* tile_start, int tokens, int hidden, int inter,
-                                           int n_experts, int top_k, int scale_stride, int ue8m0,
-                                           hipStream_t stream) {
+// h_marks / band_config (internal to the library): marks of the exact requantisation for
+// moe_requant_fix_launcher, [pairs, inter] bytes, or null; bits 10-11 of band_config scale the band.
+extern "C" void moe_gate_up_tiled_marked_launcher(void* h_q, float* h_s, float* hs_t, void* h_marks,
+                                                  const void* x_q, const float* xs_t, const void* w13_q,
+                                                  const float* w13_s, const int* sorted_pairs,
+                                                  const int* expert_offsets, const int* tile_start, int tokens,
+                                                  int hidden, int inter, int n_experts, int top_k,
+                                                  int scale_stride, int ue8m0, int band_config,
+                                                  hipStream_t stream) {
     if (tokens <= 0) return;
     if (hidden % GROUP != 0 || inter % GROUP != 0 || hidden <= 0 || inter <= 0 ||
         (unsigned long long)tokens * hidden >= (1ull << 32)) {  // 32-bit activation offsets
@@ -591,11 +648,24 @@ extern "C" void moe_gate_up_tiled_launcher(void* h_q, float* h_s, float* hs_t, c
     }
     const int max_tiles = (tokens * top_k) / TILE_PAIRS + n_experts;
     const dim3 grid(tiled_grid(inter / GROUP, max_tiles));
-    const auto kernel = ue8m0 ? moe_tiled_gemm_kernel<true, true> : moe_tiled_gemm_kernel<true, false>;
+    const auto kernel = h_marks ? (ue8m0 ? moe_tiled_gemm_kernel<true, true, true> : moe_tiled_gemm_kernel<true, false, true>)
+                                : (ue8m0 ? moe_tiled_gemm_kernel<true, true, false> : moe_tiled_gemm_kernel<true, false, false>);
     kernel<<<grid, 512, 0, stream>>>(
         static_cast<const uint8_t*>(w13_q), w13_s, static_cast<const uint8_t*>(x_q), xs_t, sorted_pairs,
         expert_offsets, tile_start, static_cast<uint8_t*>(h_q), h_s, hs_t, nullptr, hidden, 2 * inter,
-        inter, top_k, n_experts, scale_stride);
+        inter, top_k, n_experts, scale_stride, static_cast<uint8_t*>(h_marks),
+        requant_error_coefficient(band_config));
+}
+
+extern "C" void moe_gate_up_tiled_launcher(void* h_q, float* h_s, float* hs_t, const void* x_q,
+                                           const float* xs_t, const void* w13_q, const float* w13_s,
+                                           const int* sorted_pairs, const int* expert_offsets,
+                                           const int* tile_start, int tokens, int hidden, int inter,
+                                           int n_experts, int top_k, int scale_stride, int ue8m0,
+                                           hipStream_t stream) {
+    moe_gate_up_tiled_marked_launcher(h_q, h_s, hs_t, nullptr, x_q, xs_t, w13_q, w13_s, sorted_pairs,
+                                      expert_offsets, tile_start, tokens, hidden, inter, n_experts, top_k,
+                                      scale_stride, ue8m0, 0, stream);
 }
 
 extern "C" void moe_down_tiled_launcher(float* y, const void* h_q, const float* hs_t, const void* w2_q,
@@ -615,5 +685,5 @@ extern "C" void moe_down_tiled_launcher(float* y, const void* h_q, const float* 
     kernel<<<grid, 512, 0, stream>>>(
         static_cast<const uint8_t*>(w2_q), w2_s, static_cast<const uint8_t*>(h_q), hs_t, nullptr,
         expert_offsets, tile_start, nullptr, nullptr, nullptr, y, inter, hidden, inter, top_k,
-        n_experts, scale_stride);
+        n_experts, scale_stride, nullptr, 0.f);
 }

@@ -24,6 +24,19 @@ extern "C" void moe_down_launcher(float* y, const void* h_q, const float* h_s, c
                                   const float* w2_s, const int* expert_offsets, int tokens, int hidden,
                                   int inter, int n_experts, int top_k, int config, hipStream_t stream);
 
+extern "C" void moe_gate_up_tiled_marked_launcher(void* h_q, float* h_s, float* hs_t, void* h_marks,
+                                                  const void* x_q, const float* xs_t, const void* w13_q,
+                                                  const float* w13_s, const int* sorted_pairs,
+                                                  const int* expert_offsets, const int* tile_start, int tokens,
+                                                  int hidden, int inter, int n_experts, int top_k,
+                                                  int scale_stride, int ue8m0, int band_config,
+                                                  hipStream_t stream);
+extern "C" void moe_requant_fix_launcher(void* h_q, float* h_s, float* hs_t, const void* h_marks,
+                                         const void* x_q, const float* x_s, const void* w13_q,
+                                         const float* w13_s, const int* sorted_pairs,
+                                         const int* expert_offsets, int tokens, int hidden, int inter,
+                                         int n_experts, int top_k, int scale_stride, int ue8m0,
+                                         hipStream_t stream);
 extern "C" void moe_tiled_prepare_launcher(int* tile_start, float* xs_t, const float* x_s,
                                            const int* sorted_pairs, const int* expert_offsets,
                                            int tokens, int hidden, int n_experts, int top_k,
@@ -145,43 +158,71 @@ extern "C" size_t moe_fp8_workspace_bytes(int tokens, int hidden, int inter, int
 }
 
 // Byte offsets of the intermediate buffers inside the workspace, in the order
-// ids, weights, expert_offsets, sorted_pairs, pair_pos, x_q, x_s, h_q, h_s, y
+// ids, weights, expert_offsets, sorted_pairs, pair_pos, x_q, x_s, h_q, h_s, y, h_marks
 // (for checkers that compare the stages against a reference).
-extern "C" void moe_fp8_workspace_layout(size_t* offsets10, int tokens, int hidden, int inter,
+extern "C" void moe_fp8_workspace_layout(size_t* offsets11, int tokens, int hidden, int inter,
                                          int n_experts, int top_k) {
     char* base = reinterpret_cast<char*>(uintptr_t{4096});
     const moe::Workspace w = moe::carve_workspace(base, tokens, hidden, inter, n_experts, top_k);
-    const void* ptrs[10] = {w.ids, w.weights, w.expert_offsets, w.sorted_pairs, w.pair_pos,
-                            w.x_q, w.x_s,     w.h_q,            w.h_s,          w.y};
-    for (int i = 0; i < 10; ++i) offsets10[i] = static_cast<const char*>(ptrs[i]) - base;
+    const void* ptrs[11] = {w.ids, w.weights, w.expert_offsets, w.sorted_pairs, w.pair_pos, w.x_q,
+                            w.x_s, w.h_q,     w.h_s,            w.y,            w.h_marks};
+    for (int i = 0; i < 11; ++i) offsets11[i] = static_cast<const char*>(ptrs[i]) - base;
 }
 
 namespace {
 
+// How the expert GEMMs of one group of experts run: LDS-tiled or weight-streaming form, with or without the
+// exact requantisation pass. Resolved, and checked against what the chosen kernels support, before the first
+// launch of a layer, so that a shape one stage rejects launches nothing at all.
+struct GemmPlan {
+    bool ok;
+    bool tiled;
+    bool exact;
+};
+
+GemmPlan plan_expert_gemms(int tokens, int hidden, int inter, int n_experts, int top_k, int config) {
+    const int form = config & ~(CONFIG_UE8M0 | CONFIG_LAST_EXPERT_FIRST | CONFIG_REQUANT_BITS);
+    // (the tiled kernels address activations with 32-bit byte offsets and scan the tiles of at most 1024 experts)
+    const bool tiled_ok = hidden % 256 == 0 && n_experts <= 1024 &&
+                          (unsigned long long)tokens * hidden < (1ull << 32) &&
+                          (unsigned long long)tokens * top_k * inter < (1ull << 32);
+    GemmPlan plan{};
+    plan.tiled = form == 16 || (form == 0 && (long)tokens * top_k > 32L * n_experts && tiled_ok);
+    plan.ok = !plan.tiled || tiled_ok;
+    // The streaming gate/up GEMM is exact by itself (bf16 matrix core; e4m3 on request). The tiled one runs on
+    // the e4m3 matrix core and is followed by the pass that recomputes marked elements only on request: with
+    // thousands of pairs per expert that pass re-reads two weight rows for every few dozen elements of h.
+    plan.exact = plan.tiled && (config & CONFIG_EXACT_REQUANT) != 0 && !(config & CONFIG_APPROX_REQUANT);
+    if (plan.exact && hidden > 16384) plan.ok = false;
+    return plan;
+}
+
 // gate/up and down GEMMs of the experts over the quantised activations and the sort in `w`; result
 // in w.y. Many pairs per expert: LDS-tiled GEMMs (256 x 256 tiles). Few: the weight-streaming form.
-void run_expert_gemms(const moe::Workspace& w, const void* w13_q, const float* w13_s,
+void run_expert_gemms(const moe::Workspace& w, const GemmPlan& plan, const void* w13_q, const float* w13_s,
                       const void* w2_q, const float* w2_s, int tokens, int hidden, int inter,
                       int n_experts, int top_k, int config, hipStream_t stream) {
     const int ue8m0 = config & CONFIG_UE8M0;  // power-of-two block scales, see moe_fp8_launcher
     const int order = config & CONFIG_LAST_EXPERT_FIRST;
-    config &= ~(CONFIG_UE8M0 | CONFIG_LAST_EXPERT_FIRST);
-    // (the tiled kernels address activations with 32-bit byte offsets)
-    const bool fits32 = (unsigned long long)tokens * hidden < (1ull << 32) &&
-                        (unsigned long long)tokens * top_k * inter < (1ull << 32);
-    const bool tiled = config == 16 || (config == 0 && (long)tokens * top_k > 32L * n_experts &&
-                                        hidden % 256 == 0 && fits32);
-    if (tiled) {
+    const int band = config & CONFIG_BAND_MASK;
+    const int approx = config & CONFIG_APPROX_REQUANT;
+    config &= ~(CONFIG_UE8M0 | CONFIG_LAST_EXPERT_FIRST | CONFIG_REQUANT_BITS);
+    uint8_t* marks = plan.exact ? w.h_marks : nullptr;
+    if (plan.tiled) {
         moe_tiled_prepare_launcher(w.tile_start, w.xs_t, w.x_s, w.sorted_pairs, w.expert_offsets, tokens,
                                    hidden, n_experts, top_k, w.scale_stride, stream);
-        moe_gate_up_tiled_launcher(w.h_q, w.h_s, w.hs_t, w.x_q, w.xs_t, w13_q, w13_s, w.sorted_pairs,
-                                   w.expert_offsets, w.tile_start, tokens, hidden, inter, n_experts,
-                                   top_k, w.scale_stride, ue8m0, stream);
+        moe_gate_up_tiled_marked_launcher(w.h_q, w.h_s, w.hs_t, marks, w.x_q, w.xs_t, w13_q, w13_s,
+                                          w.sorted_pairs, w.expert_offsets, w.tile_start, tokens, hidden, inter,
+                                          n_experts, top_k, w.scale_stride, ue8m0, band, stream);
+        if (marks)
+            moe_requant_fix_launcher(w.h_q, w.h_s, w.hs_t, marks, w.x_q, w.x_s, w13_q, w13_s, w.sorted_pairs,
+                                     w.expert_offsets, tokens, hidden, inter, n_experts, top_k, w.scale_stride,
+                                     ue8m0, stream);
         moe_down_tiled_launcher(w.y, w.h_q, w.hs_t, w2_q, w2_s, w.expert_offsets, w.tile_start, tokens,
                                 hidden, inter, n_experts, top_k, w.scale_stride, ue8m0, stream);
     } else {
         moe_gate_up_launcher(w.h_q, w.h_s, w.x_q, w.x_s, w13_q, w13_s, w.sorted_pairs, w.expert_offsets,
-                             tokens, hidden, inter, n_experts, top_k, config | ue8m0 | order, stream);
+                             tokens, hidden, inter, n_experts, top_k, config | ue8m0 | order | approx, stream);
         moe_down_launcher(w.y, w.h_q, w.h_s, w2_q, w2_s, w.expert_offsets, tokens, hidden, inter,
                           n_experts, top_k, config | order, stream);
     }
@@ -198,6 +239,8 @@ bool layer_shape_ok(int hidden, int inter, int n_experts, int top_k, int tokens,
 // The whole layer. out [tokens, hidden] bf16 (out_dtype 0) or fp32 (out_dtype 1).
 // config: 0 = choose by the average number of pairs per expert (above 32: LDS-tiled GEMMs, else
 // weight streaming); 16 forces the tiled GEMMs; 1, 2, 4 (+8) force streaming, see moe_gate_up_launcher.
+// +256: with the tiled GEMMs, the exact requantisation pass (CONFIG_EXACT_REQUANT in moe_common.hpp; the
+// streaming gate/up GEMM is exact by itself); +512: the streaming gate/up GEMM on the e4m3 matrix core.
 // +32: all block scales are powers of two (UE8M0). The caller's weight scales must be; x and h are
 // then quantised with the smallest power-of-two scale >= amax/448, and the tiled GEMMs let the MFMA
 // apply the scales (no per-block multiply-add on the VALU).
@@ -207,7 +250,8 @@ extern "C" void moe_fp8_launcher(void* out, const void* x, const float* logits, 
                                  int inter, int n_experts, int top_k, int out_dtype, int config,
                                  hipStream_t stream) {
     if (tokens <= 0) return;
-    if (!layer_shape_ok(hidden, inter, n_experts, top_k, tokens, out_dtype)) {
+    const GemmPlan plan = plan_expert_gemms(tokens, hidden, inter, n_experts, top_k, config);
+    if (!layer_shape_ok(hidden, inter, n_experts, top_k, tokens, out_dtype) || !plan.ok) {
         caa::set_status(CAA_UNSUPPORTED_SHAPE);
         return;
     }
@@ -224,7 +268,7 @@ extern "C" void moe_fp8_launcher(void* out, const void* x, const float* logits, 
     moe_route_sort_launcher(w.ids, w.weights, w.sorted_pairs, w.pair_pos, w.expert_offsets, w.chunk_hist,
                             logits, tokens, n_experts, top_k, 0, stream);
     moe_quant_bf16_launcher(w.x_q, w.x_s, x, tokens, hidden, config & CONFIG_UE8M0, stream);
-    run_expert_gemms(w, w13_q, w13_s, w2_q, w2_s, tokens, hidden, inter, n_experts, top_k, config, stream);
+    run_expert_gemms(w, plan, w13_q, w13_s, w2_q, w2_s, tokens, hidden, inter, n_experts, top_k, config, stream);
     moe_combine_launcher(out, w.y, w.weights, w.pair_pos, tokens, hidden, top_k, out_dtype, 0, stream);
 }
 
@@ -252,8 +296,10 @@ extern "C" void moe_fp8_shared_launcher(void* out, const void* x, const float* l
                                         int shared_inter, int n_experts, int top_k, int out_dtype,
                                         int config, hipStream_t stream) {
     if (tokens <= 0) return;
+    const GemmPlan plan = plan_expert_gemms(tokens, hidden, inter, n_experts, top_k, config);
+    const GemmPlan shared_plan = plan_expert_gemms(tokens, hidden, shared_inter > 0 ? shared_inter : 1, 1, 1, config);
     if (!layer_shape_ok(hidden, inter, n_experts, top_k, tokens, out_dtype) || shared_inter <= 0 ||
-        shared_inter % GROUP != 0) {
+        shared_inter % GROUP != 0 || !plan.ok || !shared_plan.ok) {
         caa::set_status(CAA_UNSUPPORTED_SHAPE);
         return;
     }
@@ -272,12 +318,13 @@ extern "C" void moe_fp8_shared_launcher(void* out, const void* x, const float* l
     moe_route_sort_launcher(w.ids, w.weights, w.sorted_pairs, w.pair_pos, w.expert_offsets, w.chunk_hist,
                             logits, tokens, n_experts, top_k, 0, stream);
     moe_quant_bf16_launcher(w.x_q, w.x_s, x, tokens, hidden, config & CONFIG_UE8M0, stream);
-    run_expert_gemms(w, w13_q, w13_s, w2_q, w2_s, tokens, hidden, inter, n_experts, top_k, config, stream);
+    run_expert_gemms(w, plan, w13_q, w13_s, w2_q, w2_s, tokens, hidden, inter, n_experts, top_k, config, stream);
     sh.x_q = w.x_q;
     sh.x_s = w.x_s;
     moe_identity_sort_kernel<<<(tokens + 255) / 256, 256, 0, stream>>>(sh.sorted_pairs, sh.pair_pos,
                                                                       sh.expert_offsets, tokens);
-    run_expert_gemms(sh, sw13_q, sw13_s, sw2_q, sw2_s, tokens, hidden, shared_inter, 1, 1, config, stream);
+    run_expert_gemms(sh, shared_plan, sw13_q, sw13_s, sw2_q, sw2_s, tokens, hidden, shared_inter, 1, 1, config,
+                     stream);
     moe_combine_shared_launcher(out, w.y, w.weights, w.pair_pos, sh.y, tokens, hidden, top_k, out_dtype,
                                 0, stream);
 }
@@ -295,8 +342,9 @@ extern "C" void moe_fp8_fused_shared_launcher(void* out, const void* x, const fl
                                               int inter, int n_experts, int top_k, int out_dtype,
                                               int config, hipStream_t stream) {
     if (tokens <= 0) return;
+    const GemmPlan plan = plan_expert_gemms(tokens, hidden, inter, n_experts + 1, top_k + 1, config);
     if (!layer_shape_ok(hidden, inter, n_experts, top_k, tokens, out_dtype) || n_experts >= 512 ||
-        top_k >= 64 || (long)tokens * (top_k + 1) > 0x7fffffffL / 4) {
+        top_k >= 64 || (long)tokens * (top_k + 1) > 0x7fffffffL / 4 || !plan.ok) {
         caa::set_status(CAA_UNSUPPORTED_SHAPE);
         return;
     }
@@ -314,7 +362,7 @@ extern "C" void moe_fp8_fused_shared_launcher(void* out, const void* x, const fl
     moe_route_sort_launcher(w.ids, w.weights, w.sorted_pairs, w.pair_pos, w.expert_offsets, w.chunk_hist,
                             logits, tokens, n_experts, top_k, CONFIG_SHARED_SLOT, stream);
     moe_quant_bf16_launcher(w.x_q, w.x_s, x, tokens, hidden, config & CONFIG_UE8M0, stream);
-    run_expert_gemms(w, w13_q, w13_s, w2_q, w2_s, tokens, hidden, inter, n_experts + 1, top_k + 1,
+    run_expert_gemms(w, plan, w13_q, w13_s, w2_q, w2_s, tokens, hidden, inter, n_experts + 1, top_k + 1,
                      (config & ~CONFIG_LAST_EXPERT_FIRST) | CONFIG_LAST_EXPERT_FIRST, stream);
     moe_combine_launcher(out, w.y, w.weights, w.pair_pos, tokens, hidden, top_k + 1, out_dtype, 0, stream);
 }

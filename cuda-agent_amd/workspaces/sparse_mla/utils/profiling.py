@@ -11,7 +11,8 @@ profiler, so that an external profiler (``rocprofv3 --kernel-trace --stats -- py
 utils.profiling --single-run cuda_extension``) sees one forward.
 
 If the torch profiler reports no GPU events, the time falls back to HIP events around the
-timed loop (wall time on the stream, which then includes launch gaps).
+timed loop (wall time on the stream, which then includes launch gaps). Which of the two produced
+a figure is printed on a ``[timing]`` line per target in front of the result line.
 
 Run from the workspace directory: ``python3 -m utils.profiling``.
 """
@@ -75,7 +76,7 @@ def initialize_models():
     return torch_model, cuda_model, torch_inputs, cuda_inputs
 
 
-def benchmark_model(model, inputs, warmup_iters, run_iters):
+def benchmark_model(model, inputs, warmup_iters, run_iters, label="model"):
     """Mean GPU time per forward in microseconds."""
     start = torch.cuda.Event(enable_timing=True)
     stop = torch.cuda.Event(enable_timing=True)
@@ -91,10 +92,15 @@ def benchmark_model(model, inputs, warmup_iters, run_iters):
             stop.record()
             torch.cuda.synchronize()
 
-    device_us = sum(e.device_time for e in prof.events() if e.device_type.name == "CUDA")
+    device_events = [e for e in prof.events() if e.device_type.name == "CUDA"]
+    device_us = sum(e.device_time for e in device_events)
+    event_us = start.elapsed_time(stop) * 1e3
     if device_us > 0:
+        print(f"[timing] {label}: profiler device time, {len(device_events)} GPU events "
+              f"(stream time by events {event_us / run_iters:.3f}us)")
         return device_us / run_iters
-    return start.elapsed_time(stop) * 1e3 / run_iters
+    print(f"[timing] {label}: the profiler reported no GPU events, stream time by events")
+    return event_us / run_iters
 
 
 def print_results(torch_time, compile_time, cuda_time):
@@ -128,9 +134,9 @@ def main(argv=None):
 
     torch_compile_model = torch.compile(torch_model)
 
-    cuda_time = benchmark_model(cuda_model, cuda_inputs, WARMUP_ITERS, args.iters)
-    torch_time = benchmark_model(torch_model, torch_inputs, WARMUP_ITERS, args.iters)
-    compile_time = benchmark_model(torch_compile_model, torch_inputs, WARMUP_ITERS, args.iters)
+    cuda_time = benchmark_model(cuda_model, cuda_inputs, WARMUP_ITERS, args.iters, "cuda_extension")
+    torch_time = benchmark_model(torch_model, torch_inputs, WARMUP_ITERS, args.iters, "torch_baseline")
+    compile_time = benchmark_model(torch_compile_model, torch_inputs, WARMUP_ITERS, args.iters, "torch_compile")
     print_results(torch_time, compile_time, cuda_time)
 
 

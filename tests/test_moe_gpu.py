@@ -17,8 +17,12 @@ import torch
 
 from oracle import moe
 
+from moe_checks import code_steps, oracle_down, settle_disputed_codes
+
 pytestmark = pytest.mark.gpu
 TOL = 2e-2
+EXACT_REQUANT = 256   # config bit of the layer: the exact requantisation pass behind the tiled gate/up GEMM
+APPROX_REQUANT = 512  # config bit of the layer: the streaming gate/up GEMM on the e4m3 matrix core
 
 
 def make_case(dev, T, H, I, E, seed, biased=None):
@@ -97,25 +101,16 @@ def test_activation_quantisation_bit_exact(capi, dev):
     assert torch.equal(q.cpu().view(torch.uint8), want_q.view(torch.uint8))
 
 
-def oracle_down(h_q, h_s, ids, w2_q, w2_s):
-    """The oracle's down projection applied to given h codes/scales [T, k, I]."""
-    T, k, I = h_q.shape
-    y = torch.zeros(T, k, w2_q.shape[1])
-    for e in torch.unique(ids).tolist():
-        tok, slot = torch.nonzero(ids == e, as_tuple=True)
-        y[tok, slot] = moe.dequantize_groups(h_q[tok, slot], h_s[tok, slot]) @ \
-            moe.dequantize_blocks(w2_q[e], w2_s[e]).T
-    return y
-
-
 def check_layer(capi, dev, T, H, I, E, k, seed, config=0, biased=None):
     """Stage-wise parity: every stage is compared with the oracle's evaluation of that stage, the
-    floating-point stages on the kernel's own output of the stage before. The e4m3 MFMA sums a
-    128-block with about 16 significant bits (measured: |err| <= 2^-16 * sum|products|), so a
-    pre-activation differs from the oracle's in the 5th digit and about one requantised code in
-    a thousand lands on the other side of a rounding boundary (one code step, 6-12 % of that
-    element). Every stage therefore meets its bound on its own input, while end to end a few
-    isolated outputs exceed 2e-2 rms."""
+    floating-point stages on the kernel's own output of the stage before; then the layer output end to end:
+    max |error| <= 2e-2 of the output rms. The requantised codes of h must equal the oracle's except where an
+    fp32 evaluation is itself undecided (settle_disputed_codes): a handful per million. (The e4m3 matrix core
+    alone, which sums a 128-block with about 16 significant bits, would put about one code in a thousand on
+    the other side of a rounding boundary and move isolated outputs by 2-4 % of the rms; the streaming gate/up
+    GEMM therefore runs on the bf16 matrix core and the tiled one is followed by the exact requantisation
+    pass when config bit 256 asks for it, as every tiled case here does.)"""
+    config |= EXACT_REQUANT   # (only the tiled form looks at it)
     x, logits, w, dts = make_case(dev, T, H, I, E, seed, biased)
     w13_q, w13_s, w2_q, w2_s = w
     ref, mid = moe.moe_forward(x, logits, *w, top_k=k, out_dtype=torch.float32, return_intermediates=True)
@@ -132,10 +127,10 @@ def check_layer(capi, dev, T, H, I, E, k, seed, config=0, biased=None):
     pos = pos.long()
     hq = views['h_q'].cpu()[pos].reshape(T, k, I)
     hs = views['h_s'].cpu()[pos].reshape(T, k, I // 128)
-    torch.testing.assert_close(hs, mid['h_s'], rtol=1e-3, atol=0)
-    code_diff = (hq.view(torch.uint8).int() - mid['h_q'].view(torch.uint8).int()).abs()
-    assert (code_diff > 0).float().mean().item() < 3e-3
-    assert (code_diff > 1).float().mean().item() < 1e-4      # never more than one code step
+    torch.testing.assert_close(hs, mid['h_s'], rtol=1e-5, atol=0)
+    code_diff = code_steps(hq, mid['h_q'])
+    assert (code_diff > 0).float().mean().item() < 2e-4
+    assert not (code_diff > 1).any()                         # never more than one code step
     # down projection, on the kernel's own h
     y = views['y'].cpu()[pos].reshape(T, k, H)
     assert moe.rel_rms_error(y, oracle_down(hq, hs, mid['ids'], w2_q, w2_s)) <= 1e-3
@@ -144,17 +139,13 @@ def check_layer(capi, dev, T, H, I, E, k, seed, config=0, biased=None):
     for j in range(k):
         want += mid['weights'][:, j:j + 1] * y[:, j]
     assert moe.rel_rms_error(exact.cpu(), want) <= 1e-5
-    # end to end: requantisation is discontinuous, so the one-in-a-thousand codes that fall on the
-    # other side of a rounding boundary (see the docstring) move isolated outputs by a few
-    # percent of the rms. Bounds: rms error 0.5 %, at most 1 output in 1000 beyond 2e-2 rms,
-    # none beyond 6e-2 rms; where no code differs the plain 2e-2 bound applies.
-    diff = (exact.cpu() - ref).double().abs()
-    rms = ref.double().pow(2).mean().sqrt()
-    assert (diff.pow(2).mean().sqrt() / rms).item() <= 5e-3
-    assert (diff > TOL * rms).double().mean().item() <= 1e-3
-    assert (diff.max() / rms).item() <= 3 * TOL
-    if not (code_diff > 0).any():
-        assert (diff.max() / rms).item() <= TOL
+    # end to end
+    n_disputed, settled = settle_disputed_codes(hq, mid, w13_q, w13_s, w2_q, w2_s, k)
+    err, err_settled = moe.rel_rms_error(exact.cpu(), ref), moe.rel_rms_error(exact.cpu(), settled)
+    print(f'[moe] T={T} H={H} I={I} E={E} k={k} config={config}: {n_disputed} of {hq.numel()} h codes differ from '
+          f'the oracle (all undecided in fp32), end-to-end max error {err:.2e} of the output rms, '
+          f'{err_settled:.2e} with those codes settled')
+    assert err_settled <= TOL
     out, _ = run_layer(capi, dts, k, config)
     assert torch.equal(out, exact.bfloat16())
     return out.cpu(), ref
@@ -177,9 +168,9 @@ def test_layer_tiled_gemms(capi, dev, shape):
 @pytest.mark.parametrize('seed', range(8))
 def test_tiled_and_streaming_forms_agree_on_random_shapes(capi, dev, seed):
     # Random sizes and routing skews: experts with no pairs, with a few, with several 256-pair tiles;
-    # 1 to 7 K blocks in either GEMM. The integer stages must be identical, the codes of h may
-    # differ by one step in a few places (different summation order inside a 128 block), the outputs
-    # agree within the end-to-end bound.
+    # 1 to 7 K blocks in either GEMM. The integer stages must be identical; the codes of h (tiled GEMMs + exact
+    # requantisation pass against the streaming GEMMs on the bf16 matrix core) may differ where fp32 itself is
+    # undecided; each output meets the end-to-end bound against the oracle with such codes settled.
     rng = torch.Generator().manual_seed(1000 + seed)
     pick = lambda xs: xs[int(torch.randint(len(xs), (1,), generator=rng))]
     H, I = pick([256, 512, 768]), pick([128, 256, 384, 896])
@@ -188,34 +179,54 @@ def test_tiled_and_streaming_forms_agree_on_random_shapes(capi, dev, seed):
     T = pick([1, 37, 300, 1100])
     hot = torch.randperm(E, generator=rng)[:max(1, E // 4)] if seed % 2 else None
     x, logits, w, dts = make_case(dev, T, H, I, E, 2000 + seed, hot)
-    a, va = run_layer(capi, dts, k, 16, torch.float32)   # LDS-tiled GEMMs
-    b, vb = run_layer(capi, dts, k, 4, torch.float32)    # streaming GEMMs
+    a, va = run_layer(capi, dts, k, 16 | EXACT_REQUANT, torch.float32)   # LDS-tiled GEMMs
+    b, vb = run_layer(capi, dts, k, 4, torch.float32)                    # streaming GEMMs
     for name in ('ids', 'sorted_pairs', 'pair_pos', 'expert_offsets', 'x_s'):
         assert torch.equal(va[name], vb[name]), name
     assert torch.equal(va['x_q'].view(torch.uint8), vb['x_q'].view(torch.uint8))
-    ha = va['h_q'].view(torch.uint8).cpu()
-    hb = vb['h_q'].view(torch.uint8).cpu()
-    assert (ha != hb).float().mean().item() < 5e-3
+    assert (va['h_q'].view(torch.uint8) != vb['h_q'].view(torch.uint8)).float().mean().item() < 2e-4
     assert torch.isfinite(a).all() and torch.isfinite(b).all()
-    ref = moe.moe_forward(x, logits, *w, top_k=k, out_dtype=torch.float32)
-    rms = ref.double().pow(2).mean().sqrt()
-    for got, want in ((a.cpu(), ref), (b.cpu(), ref), (a.cpu(), b.cpu())):   # the end-to-end bounds of check_layer
-        diff = (got - want).double().abs()
-        assert (diff.pow(2).mean().sqrt() / rms).item() <= 5e-3
-        assert (diff > TOL * rms).double().mean().item() <= 1e-3
-        # one flipped code moves an output by up to 12 % of |h_j| * |w_ij|, which for inter = 128 and
-        # a single expert per token is several percent of the output rms
-        assert (diff.max() / rms).item() <= 0.15
+    ref, mid = moe.moe_forward(x, logits, *w, top_k=k, out_dtype=torch.float32, return_intermediates=True)
+    pos = va['pair_pos'].cpu().long()
+    for got, views in ((a, va), (b, vb)):
+        hq = views['h_q'].cpu()[pos].reshape(T, k, I)
+        _, settled = settle_disputed_codes(hq, mid, *w, k)
+        assert moe.rel_rms_error(got.cpu(), settled) <= TOL
+
+
+def test_requantisation_on_the_e4m3_matrix_core_is_what_the_exact_forms_remove(capi, dev):
+    # The same layer three ways: streaming gate/up on the e4m3 matrix core (config bit 512), on the bf16 one
+    # (default), and tiled GEMMs without and with the exact pass. The e4m3 forms differ from the oracle in about
+    # one code of h in a thousand, the exact forms in none or a few per million.
+    T, H, I, E, k = 300, 512, 256, 4, 2
+    x, logits, w, dts = make_case(dev, T, H, I, E, 350)
+    _, mid = moe.moe_forward(x, logits, *w, top_k=k, out_dtype=torch.float32, return_intermediates=True)
+    rate = {}
+    for name, config in (('stream e4m3', 4 | APPROX_REQUANT), ('stream bf16', 4), ('tiled', 16),
+                         ('tiled exact', 16 | EXACT_REQUANT)):
+        _, views = run_layer(capi, dts, k, config, torch.float32)
+        hq = views['h_q'].cpu()[views['pair_pos'].cpu().long()].reshape(T, k, I)
+        rate[name] = (code_steps(hq, mid['h_q']) > 0).float().mean().item()
+    print('[moe] h codes that differ from the oracle:', {n: f'{r * 1e6:.0f} ppm' for n, r in rate.items()})
+    assert 3e-4 < rate['stream e4m3'] < 3e-3 and 3e-4 < rate['tiled'] < 3e-3
+    assert rate['stream bf16'] < 1e-4 and rate['tiled exact'] < 1e-4
 
 
 def test_tiled_path_is_chosen_for_many_pairs_per_expert(capi, dev):
     # 1200 pairs over 8 experts: config 0 takes the tiled form; it must agree with streaming
     x, logits, w, dts = make_case(dev, 600, 512, 256, 8, 61)
     a, _ = run_layer(capi, dts, 2, 0, torch.float32)
-    b, _ = run_layer(capi, dts, 2, 4, torch.float32)
     c, _ = run_layer(capi, dts, 2, 16, torch.float32)
     assert torch.equal(a, c)
-    assert moe.rel_rms_error(a.cpu(), b.cpu()) <= TOL
+    a, va = run_layer(capi, dts, 2, EXACT_REQUANT, torch.float32)
+    b, vb = run_layer(capi, dts, 2, 4, torch.float32)
+    c, _ = run_layer(capi, dts, 2, 16 | EXACT_REQUANT, torch.float32)
+    assert torch.equal(a, c)
+    assert (va['h_q'].view(torch.uint8) != vb['h_q'].view(torch.uint8)).float().mean().item() < 2e-4
+    _, mid = moe.moe_forward(x, logits, *w, top_k=2, out_dtype=torch.float32, return_intermediates=True)
+    hq = va['h_q'].cpu()[va['pair_pos'].cpu().long()].reshape(600, 2, 256)
+    _, settled = settle_disputed_codes(hq, mid, *w, 2)
+    assert moe.rel_rms_error(a.cpu(), settled) <= TOL
 
 
 def test_layer_ragged_expert_load(capi, dev):
@@ -273,35 +284,194 @@ def test_decode_workload_shape_reduced_experts(capi, dev):
 
 def test_full_decode_workload_properties(capi, dev):
     """Config 2 at full size (256 experts, 11.3 GB of weights) through size-independent
-    properties: integer stages against the oracle, linearity of the layer in a routing weight,
-    and agreement of a 4-token slice with the oracle evaluated on just the experts it uses."""
+    properties: integer stages against the oracle, all outputs finite, and eight tokens against the oracle
+    evaluated on just the experts they use (stage-wise and end to end, check_sampled_tokens)."""
     T, H, I, E, k = 64, 7168, 2048, 256, 8
-    gen = torch.Generator(device=dev).manual_seed(20252)
-    w13_q = (torch.randn(E, 2 * I, H, device=dev, generator=gen) * (448 / H ** 0.5)).to(torch.float8_e4m3fn)
-    w2_q = (torch.randn(E, H, I, device=dev, generator=gen) * (448 / I ** 0.5)).to(torch.float8_e4m3fn)
-    w13_s = (0.5 + torch.rand(E, 2 * I // 128, H // 128, device=dev, generator=gen)) / 448
-    w2_s = (0.5 + torch.rand(E, H // 128, I // 128, device=dev, generator=gen)) / 448
-    x = torch.randn(T, H, device=dev, generator=gen).bfloat16()
-    logits = torch.randn(T, E, device=dev, generator=gen)
-    dts = [x, logits, w13_q, w13_s, w2_q, w2_s]
+    dts = full_size_layer(dev, T, 20252)
+    x, logits = dts[0], dts[1]
     exact, views = run_layer(capi, dts, k, 0, torch.float32)
     ids, _ = moe.route(logits.cpu(), k)
     assert torch.equal(views['ids'].cpu(), ids)
     sp, pos, off = moe.sort_pairs(ids, E)
     assert torch.equal(views['sorted_pairs'].cpu(), sp) and torch.equal(views['expert_offsets'].cpu(), off)
-    # tokens 0..3 against the oracle restricted to their experts (weights copied to the host)
-    used = torch.unique(ids[:4]).tolist()
-    remap = {e: i for i, e in enumerate(used)}
-    sub_logits = torch.full((4, len(used)), -30.0)
-    for t in range(4):
-        for e in ids[t].tolist():
-            sub_logits[t, remap[e]] = logits[t, e].item()
-    sel = torch.tensor(used, device=dev)
-    ref = moe.moe_forward(x[:4].cpu(), sub_logits, w13_q[sel].cpu(), w13_s[sel].cpu(), w2_q[sel].cpu(),
-                          w2_s[sel].cpu(), top_k=k, out_dtype=torch.float32)
-    # routing weights are sigmoid ratios over the same 8 logits, so the restriction changes nothing
-    assert moe.rel_rms_error(exact[:4].cpu(), ref) <= 3 * TOL
+    x_q, x_s = moe.quantize_groups(x.cpu().float())
+    assert torch.equal(views['x_q'].cpu().view(torch.uint8), x_q.view(torch.uint8))
+    assert torch.equal(views['x_s'].cpu(), x_s)
     assert torch.isfinite(exact).all()
+    check_sampled_tokens(list(range(0, 64, 8)), dts, ids, pos, views, exact, k)
+    out, _ = run_layer(capi, dts, k, 0)
+    assert torch.equal(out, exact.bfloat16())
+
+
+def full_size_layer(dev, T, seed, n_biased=0):
+    """Workload-sized layer (hidden 7168, intermediate 2048, 256 experts, 11.3 GB of weights) drawn on
+    the device; the logits of ``n_biased`` experts chosen by a seeded permutation are raised by 2."""
+    H, I, E = 7168, 2048, 256
+    gen = torch.Generator(device=dev).manual_seed(seed)
+    w13_q = torch.empty(E, 2 * I, H, dtype=torch.float8_e4m3fn, device=dev)
+    w2_q = torch.empty(E, H, I, dtype=torch.float8_e4m3fn, device=dev)
+    for e0 in range(0, E, 32):                       # 32 experts at a time: the fp32 draw stays at 3.8 GB
+        w13_q[e0:e0 + 32] = (torch.randn(32, 2 * I, H, device=dev, generator=gen) * (448 / H ** 0.5)) \
+            .clamp(-448, 448).to(torch.float8_e4m3fn)
+        w2_q[e0:e0 + 32] = (torch.randn(32, H, I, device=dev, generator=gen) * (448 / I ** 0.5)) \
+            .clamp(-448, 448).to(torch.float8_e4m3fn)
+    w13_s = (0.5 + torch.rand(E, 2 * I // 128, H // 128, device=dev, generator=gen)) / 448
+    w2_s = (0.5 + torch.rand(E, H // 128, I // 128, device=dev, generator=gen)) / 448
+    x = torch.randn(T, H, device=dev, generator=gen).bfloat16()
+    logits = torch.randn(T, E, device=dev, generator=gen)
+    if n_biased:
+        hot = torch.randperm(E, generator=torch.Generator().manual_seed(seed))[:n_biased]
+        logits[:, hot.to(dev)] += 2.0
+    return [x, logits, w13_q, w13_s, w2_q, w2_s]
+
+
+def oracle_on_tokens(tokens, dts, ids, k):
+    """The oracle layer on the given tokens, evaluated over just the experts they use (their weights
+    copied to the host). Routing weights are ratios of sigmoids of a token's own 8 logits, so leaving
+    the other experts out changes nothing. Returns (out fp32, intermediates with global expert ids)."""
+    x, logits, w13_q, w13_s, w2_q, w2_s = dts
+    tokens = torch.as_tensor(tokens)
+    used = torch.unique(ids[tokens]).tolist()
+    remap = {e: i for i, e in enumerate(used)}
+    sub_logits = torch.full((len(tokens), len(used)), -30.0)
+    host_logits = logits[tokens.to(logits.device)].cpu()
+    for r, t in enumerate(tokens.tolist()):
+        for e in ids[t].tolist():
+            sub_logits[r, remap[e]] = host_logits[r, e]
+    sel = torch.tensor(used, device=x.device)
+    w = [t[sel].cpu() for t in (w13_q, w13_s, w2_q, w2_s)]
+    ref, mid = moe.moe_forward(x[tokens.to(x.device)].cpu(), sub_logits, *w, top_k=k, out_dtype=torch.float32,
+                               return_intermediates=True)
+    back = torch.tensor(used, dtype=torch.int32)
+    assert torch.equal(back[mid['ids'].long()], ids[tokens])
+    mid['local_ids'], mid['ids'], mid['w'] = mid['ids'], ids[tokens], w
+    return ref, mid
+
+
+def check_sampled_tokens(tokens, dts, ids, pos, views, exact, k, exact_requant=True):
+    """The stage-wise and end-to-end bounds of check_layer for a sample of tokens of a full-size layer.
+    exact_requant False: the layer ran the tiled GEMMs without the exact requantisation pass, so about one h
+    code in a thousand is one step off and the end-to-end error is reported, and bounded by 3x the tolerance,
+    instead of by the tolerance."""
+    H, I = dts[0].shape[1], dts[2].shape[1] // 2
+    ref, mid = oracle_on_tokens(tokens, dts, ids, k)
+    w13_q, w13_s, w2_q, w2_s = mid['w']
+    tokens = torch.as_tensor(tokens)
+    rows = pos.long().reshape(-1, k)[tokens].reshape(-1).to(exact.device)       # sorted positions of their pairs
+    n = len(tokens)
+    hq = views['h_q'].view(torch.uint8)[rows].cpu().view(torch.float8_e4m3fn).reshape(n, k, I)
+    hs = views['h_s'][rows].cpu().reshape(n, k, I // 128)
+    torch.testing.assert_close(hs, mid['h_s'], rtol=1e-5 if exact_requant else 1e-3, atol=0)
+    code_diff = code_steps(hq, mid['h_q'])
+    flips = (code_diff > 0).float().mean().item()
+    assert flips < (2e-4 if exact_requant else 3e-3)
+    # (on the e4m3 matrix core a value near zero, where the format's steps are 2^-9 of the scale, can be two
+    # steps off: its error is absolute, about 1e-5 of the rms of the pre-activations)
+    far = code_diff > 1
+    if far.any():
+        table = torch.from_numpy(moe.e4m3_decode_table())
+        print(f'[moe] {int(far.sum())} of {hq.numel()} h codes more than one step off, at most {int(code_diff.max())} steps, '
+              f'largest magnitude among them {table[(mid["h_q"].view(torch.uint8)[far] & 0x7f).long()].max().item()} of 448')
+    assert not far.any() if exact_requant else far.float().mean().item() < 1e-4
+    y = views['y'][rows].cpu().reshape(n, k, H)
+    local = dict(mid, ids=mid['local_ids'])
+    assert moe.rel_rms_error(y, oracle_down(hq, hs, mid['local_ids'], w2_q, w2_s)) <= 1e-3
+    want = torch.zeros(n, H)
+    for j in range(k):
+        want += mid['weights'][:, j:j + 1] * y[:, j]
+    got = exact[tokens.to(exact.device)].cpu()
+    assert moe.rel_rms_error(got, want) <= 1e-5
+    err = moe.rel_rms_error(got, ref)
+    if exact_requant:
+        n_disputed, settled = settle_disputed_codes(hq, local, w13_q, w13_s, w2_q, w2_s, k)
+        err_settled = moe.rel_rms_error(got, settled)
+        print(f'[moe] {n} sampled tokens: {n_disputed} of {hq.numel()} h codes differ from the oracle (all undecided '
+              f'in fp32), end-to-end max error {err:.2e} of the output rms, {err_settled:.2e} with those settled')
+        assert err_settled <= TOL
+    else:
+        beyond = ((got - ref).abs() > TOL * ref.double().pow(2).mean().sqrt()).float().mean().item()
+        print(f'[moe] {n} sampled tokens, e4m3 matrix core without the exact pass: {flips * 1e3:.2f} per mille of h '
+              f'codes one step off, end-to-end max error {err:.2e} of the output rms, {beyond * 1e6:.0f} ppm of '
+              f'the outputs beyond {TOL}')
+        assert err <= 3 * TOL and beyond <= 1e-3
+    return err
+
+
+def test_full_prefill_workload_properties(capi, dev):
+    """Config 4 at full size (8192 tokens, 256 experts, +2 on the logits of 16 experts). The integer stages and
+    the activation codes against the oracle at full size. The floating-point stages and the end-to-end bound
+    against the oracle on sampled tokens that sit in the first, a middle and the ragged last 256-pair tile of
+    the most loaded expert and in the first and last pair of four lightly loaded experts: for the layer as it
+    runs by default at this size (tiled GEMMs on the e4m3 matrix core: the deviation is printed and bounded by
+    3x the tolerance), and with the exact requantisation pass (the stated tolerance). The whole output against
+    the weight-streaming form of the layer (separately written kernels); all outputs finite; the bf16 output
+    equal to the rounding of the fp32 one."""
+    T, H, I, E, k = 8192, 7168, 2048, 256, 8
+    dts = full_size_layer(dev, T, 20254, n_biased=16)
+    x, logits = dts[0], dts[1]
+    exact, views = run_layer(capi, dts, k, 0, torch.float32)       # config 0 must take the tiled GEMMs
+    ids, weights = moe.route(logits.cpu(), k)
+    assert torch.equal(views['ids'].cpu(), ids)
+    torch.testing.assert_close(views['weights'].cpu(), weights, rtol=1e-6, atol=1e-7)
+    sp, pos, off = moe.sort_pairs(ids, E)
+    assert torch.equal(views['sorted_pairs'].cpu(), sp) and torch.equal(views['pair_pos'].cpu(), pos)
+    assert torch.equal(views['expert_offsets'].cpu(), off)
+    x_q, x_s = moe.quantize_groups(x.cpu().float())
+    assert torch.equal(views['x_q'].cpu().view(torch.uint8), x_q.view(torch.uint8))
+    assert torch.equal(views['x_s'].cpu(), x_s)
+    assert torch.isfinite(exact).all()
+
+    counts = (off[1:] - off[:-1]).long()
+    hot = int(counts.argmax())
+    n_hot = int(counts[hot])
+    assert n_hot > 4 * 256 and n_hot % 256 != 0, 'the most loaded expert should have several tiles and a ragged one'
+    last_tile = (n_hot - 1) // 256 * 256
+    sample_pos = [off[hot] + p for p in (0, 255, (n_hot // 512) * 256 + 77, last_tile, n_hot - 1)]
+    cold = [int(e) for e in torch.argsort(counts)[:60:15]]          # four of the lightly loaded experts
+    assert all(0 < counts[e] < 256 for e in cold)
+    for e in cold:
+        sample_pos += [off[e], off[e + 1] - 1]
+    tokens = sorted({int(sp[int(p)]) // k for p in sample_pos})
+    more = torch.randperm(T, generator=torch.Generator().manual_seed(4))[:16 - len(tokens)].tolist()
+    tokens = sorted(set(tokens) | set(more))
+    assert len(tokens) >= 12
+    check_sampled_tokens(tokens, dts, ids, pos, views, exact, k, exact_requant=False)
+    out, _ = run_layer(capi, dts, k, 0)
+    assert torch.equal(out, exact.bfloat16())
+    del out, views
+
+    # the same tiles with the exact requantisation pass behind the gate/up GEMM: the stated tolerance
+    fixed, views = run_layer(capi, dts, k, EXACT_REQUANT, torch.float32)
+    assert torch.isfinite(fixed).all()
+    check_sampled_tokens(tokens, dts, ids, pos, views, fixed, k)
+    marks = views['h_marks']
+    print(f'[moe] exact requantisation at full size: {(marks & 1).float().mean().item() * 100:.2f} % of the elements '
+          f'of h recomputed for their code, {((marks >> 1) & 1).float().mean().item() * 100:.2f} % as candidates '
+          f'for the maximum of their group')
+    hq_fixed = views['h_q'].clone()
+    del views, marks
+    # what leaving the pass out (the default at this size) does to the whole output
+    rms = fixed.double().pow(2).mean().sqrt()
+    diff = (exact - fixed).abs()
+    beyond = (diff > TOL * rms).float().mean().item()
+    print(f'[moe] tiled GEMMs without against with the exact pass at full size: rms difference '
+          f'{(diff.double().pow(2).mean().sqrt() / rms).item():.2e} of the output rms, max '
+          f'{(diff.max().double() / rms).item():.2e}, {beyond * 1e6:.2f} ppm of the outputs beyond {TOL}')
+    assert (diff.max().double() / rms).item() <= 3 * TOL and beyond <= 1e-4
+    del exact
+
+    # the same layer through the weight-streaming GEMMs (gate/up on the bf16 matrix core): same integer stages;
+    # h codes differ only where fp32 is undecided; such a difference on a large element still moves single
+    # outputs by a few percent of the rms, so the whole outputs are compared by their rms difference and by
+    # the share of outputs beyond the tolerance
+    streamed, views_s = run_layer(capi, dts, k, 4, torch.float32)
+    assert (views_s['h_q'].view(torch.uint8) != hq_fixed.view(torch.uint8)).float().mean().item() < 2e-4
+    diff = (streamed - fixed).abs()
+    gap_rms = (diff.double().pow(2).mean().sqrt() / rms).item()
+    beyond = (diff > TOL * rms).float().mean().item()
+    print(f'[moe] tiled + exact pass against streaming form at full size: rms difference {gap_rms:.2e} of the output '
+          f'rms, max {(diff.max().double() / rms).item():.2e}, {beyond * 1e6:.2f} ppm of the outputs beyond {TOL}')
+    assert gap_rms <= 1e-3 and beyond <= 1e-5
 
 
 def test_rejects_bad_arguments(capi, dev):

@@ -14,6 +14,8 @@ import torch
 
 from oracle import moe
 
+from moe_checks import code_steps, settle_disputed_codes
+
 pytestmark = pytest.mark.gpu
 TOL = 2e-2
 UE8M0 = 32
@@ -111,6 +113,25 @@ def check_layer(capi, dev, T, H, I, E, k, seed, config, biased=None):
 def test_layer(capi, dev, shape, config):
     T, H, I, E, k = shape
     check_layer(capi, dev, T, H, I, E, k, seed=70 + T, config=config)
+
+
+@pytest.mark.parametrize('config', [16 | 256, 4])
+@pytest.mark.parametrize('shape', [(300, 512, 256, 4, 2), (520, 768, 384, 3, 3)])
+def test_layer_with_exact_requantisation(capi, dev, shape, config):
+    # the forms whose h agrees with an fp32 evaluation: tiled GEMMs followed by the exact requantisation pass
+    # (config bit 256) and streaming GEMMs (gate/up on the bf16 matrix core): the scales are the oracle's, the
+    # codes differ only where fp32 is undecided, the output meets the plain end-to-end bound
+    T, H, I, E, k = shape
+    x, logits, w, dts = make_case(dev, T, H, I, E, 70 + T)
+    ref, mid = moe.moe_forward(x, logits, *w, top_k=k, out_dtype=torch.float32, return_intermediates=True,
+                               pow2_scales=True)
+    exact, views = run_layer(capi, dts, k, config)
+    pos = moe.sort_pairs(mid['ids'], E)[1].long()
+    hq = views['h_q'].cpu()[pos].reshape(T, k, I)
+    assert torch.equal(views['h_s'].cpu()[pos].reshape(T, k, I // 128), mid['h_s'])
+    assert (code_steps(hq, mid['h_q']) > 0).float().mean().item() < 2e-4
+    _, settled = settle_disputed_codes(hq, mid, *w, k)
+    assert moe.rel_rms_error(exact.cpu(), settled) <= TOL
 
 
 def test_tiled_and_streaming_forms_agree(capi, dev):
