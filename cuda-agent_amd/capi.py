@@ -36,6 +36,9 @@ SIGNATURES = {
                                                     _P]),
     'sparse_mla_decode_num_splits': (c_int, [c_int, c_int, c_int, c_int]),
     'sparse_mla_decode_workspace_bytes': (c_size_t, [c_int, c_int, c_int, c_int]),
+    'sparse_mla_decode_static_scratch_bytes': (c_size_t, []),
+    'sparse_mla_decode_static_launcher': (None, [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
+                                                 c_int, c_int, _P]),
     'mla_latent_quant_launcher': (None, [_P, _P, c_long, c_int, _P]),
     'sparse_mla_decode_fp8_workspace_bytes': (c_size_t, [c_int, c_int, c_int, c_int]),
     'sparse_mla_decode_fp8_launcher': (None, [_P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int,
@@ -75,7 +78,8 @@ SIGNATURES = {
                                 c_int, c_int, c_int, _P]),
 }
 
-STATUS_NAMES = {0: 'ok', 1: 'unsupported shape', 2: 'bad argument', 3: 'workspace too small'}
+STATUS_NAMES = {0: 'ok', 1: 'unsupported shape', 2: 'bad argument', 3: 'workspace too small',
+                4: 'more scratch needed than the static array holds', 5: 'HIP runtime error during set-up'}
 
 _lib = None
 
@@ -267,6 +271,27 @@ def sparse_mla_decode_launch(out, q, kv, idx, workspace, sm_scale=192 ** -0.5, c
                                          0 if out.dtype == torch.bfloat16 else 1, config,
                                          _stream(stream))
     check_status('sparse_mla_decode_launcher')
+    return out
+
+
+def sparse_mla_decode_static_launch(out, q, kv, idx, sm_scale=192 ** -0.5, config=0, stream=None):
+    """sparse_mla_decode_launch without a workspace: the split partials go to the library's static device array
+    (``sparse_mla_decode_static_scratch_bytes()``); nothing is allocated. Calls that overlap on one GPU race."""
+    import torch
+    _device_contiguous(out=out, q=q, kv=kv, idx=idx)
+    B, H, d_qk = q.shape
+    N = kv.shape[1]
+    topk = idx.shape[1]
+    d_v = out.shape[2]
+    _require(q.dtype == kv.dtype == torch.bfloat16, 'sparse_mla: q, kv must be bf16')
+    _require(out.dtype in (torch.bfloat16, torch.float32), 'sparse_mla: out must be bf16 or fp32')
+    _require(idx.dtype == torch.int32, 'sparse_mla: idx must be int32')
+    _require(tuple(kv.shape) == (B, N, d_qk) and tuple(idx.shape) == (B, topk), 'sparse_mla: kv/idx shape')
+    _require(tuple(out.shape) == (B, H, d_v), 'sparse_mla: out shape')
+    library().sparse_mla_decode_static_launcher(_ptr(out), _ptr(q), _ptr(kv), _ptr(idx), B, H, N, topk, d_qk, d_v,
+                                                float(sm_scale), 0 if out.dtype == torch.bfloat16 else 1, config,
+                                                _stream(stream))
+    check_status('sparse_mla_decode_static_launcher')
     return out
 
 

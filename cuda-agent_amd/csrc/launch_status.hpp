@@ -11,6 +11,8 @@ enum CudaAgentAmdStatus : int {
     CAA_UNSUPPORTED_SHAPE = 1,   // a dimension the kernels are not instantiated for
     CAA_BAD_ARGUMENT = 2,        // null pointer, misaligned base, negative size
     CAA_WORKSPACE_TOO_SMALL = 3, // caller-provided scratch is smaller than *_workspace_bytes()
+    CAA_SCRATCH_LIMIT = 4,       // the problem needs more than the library's own static scratch holds
+    CAA_RUNTIME_ERROR = 5,       // a HIP runtime call of the launcher's set-up failed
 };
 
 namespace caa {

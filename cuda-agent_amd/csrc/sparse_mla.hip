@@ -34,6 +34,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "launch_status.hpp"
 #include "mla_addressing.hpp"
 
@@ -1278,6 +1280,67 @@ extern "C" void sparse_mla_decode_paged_launcher(void* out, const void* q, const
     const KvAddressing kva{block_table, max_pages_per_request, page_shift, 0};
     launch_sparse_mla(out, q, kv_pool, idx, workspace, workspace_bytes, batch, n_heads,
                       n_pages * page_size, topk, d_qk, d_v, sm_scale, out_dtype, config, kva, stream);
+}
+
+// ---- the entry point that allocates nothing ------------------------------------------------------------------
+// Scratch of sparse_mla_decode_static_launcher: the partial outputs of the key splits live in this array of the
+// library's own instead of in a caller-provided workspace. Every GPU the library runs on holds one copy from
+// module load to process end. 72 MiB covers 64 requests x 128 heads x 2048 selected rows in 4 splits
+// (67 371 008 bytes) with some room.
+constexpr size_t STATIC_SCRATCH_BYTES = (size_t)72 << 20;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+namespace {
+
+constexpr int MAX_SCRATCH_DEVICES = 64;
+std::atomic<void*> g_scratch_ptr[MAX_SCRATCH_DEVICES];  // device address of `scratch` on every device, once known
+
+// Device address of this device's copy of `scratch` (the array's name is a host-side stand-in, not an address a
+// kernel could use). Looked up once per device, with that device current; null on failure.
+void* static_scratch() {
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= MAX_SCRATCH_DEVICES) return nullptr;
+    void* ptr = g_scratch_ptr[device].load(std::memory_order_acquire);
+    if (ptr == nullptr) {
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) return nullptr;
+        g_scratch_ptr[device].store(ptr, std::memory_order_release);  // (a concurrent first call stores the same value)
+    }
+    return ptr;
+}
+
+}  // namespace
+
+// sparse_mla_decode_launcher for callers that cannot allocate device memory (code under HIP graph capture,
+// serving loops with a fixed memory plan, harnesses that forbid it): same arguments without the workspace, same
+// kernels, same result bit for bit. The split partials go to a static device array of STATIC_SCRATCH_BYTES.
+// Limits and rules that follow from that:
+//   * sparse_mla_decode_workspace_bytes(batch, n_heads, topk, config) must not exceed
+//     sparse_mla_decode_static_scratch_bytes(); a larger problem is rejected (status CAA_SCRATCH_LIMIT) and
+//     nothing is launched;
+//   * all calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two streams, two
+//     threads) race; calls on one stream are ordered and safe. Nothing in the array has to start at zero (every
+//     partial the merge reads was written by the split kernel of the same call), so it is never cleared;
+//   * the first call on a device looks up the array's device address (hipGetSymbolAddress): make that call
+//     outside a graph capture. No call allocates or frees memory.
+extern "C" size_t sparse_mla_decode_static_scratch_bytes(void) { return STATIC_SCRATCH_BYTES; }
+
+extern "C" void sparse_mla_decode_static_launcher(void* out, const void* q, const void* kv, const int* idx,
+                                                  int batch, int n_heads, int n_kv_rows, int topk, int d_qk,
+                                                  int d_v, float sm_scale, int out_dtype, int config,
+                                                  hipStream_t stream) {
+    if (batch <= 0 || n_heads <= 0 || topk <= 0) return;
+    if (sparse_mla_decode_workspace_bytes(batch, n_heads, topk, config) > STATIC_SCRATCH_BYTES) {
+        caa::set_status(CAA_SCRATCH_LIMIT);
+        return;
+    }
+    void* ptr = static_scratch();
+    if (ptr == nullptr) {
+        caa::set_status(CAA_RUNTIME_ERROR);
+        return;
+    }
+    const KvAddressing kva{nullptr, 0, 0, n_kv_rows};
+    launch_sparse_mla(out, q, kv, idx, ptr, STATIC_SCRATCH_BYTES, batch, n_heads, n_kv_rows, topk, d_qk, d_v,
+                      sm_scale, out_dtype, config, kva, stream);
 }
 
 // Decode over a cache in the 656-byte e4m3 form with the dequantisation inside the 128-head kernel (see

@@ -40,7 +40,9 @@ enum {
     CUDA_AGENT_AMD_OK = 0,
     CUDA_AGENT_AMD_UNSUPPORTED_SHAPE = 1,
     CUDA_AGENT_AMD_BAD_ARGUMENT = 2,
-    CUDA_AGENT_AMD_WORKSPACE_TOO_SMALL = 3
+    CUDA_AGENT_AMD_WORKSPACE_TOO_SMALL = 3,
+    CUDA_AGENT_AMD_SCRATCH_LIMIT = 4, /* more scratch needed than the library's static array holds */
+    CUDA_AGENT_AMD_RUNTIME_ERROR = 5  /* a HIP runtime call of a launcher's set-up failed */
 };
 
 /* Code of the calling thread's most recent rejected launch since the last query; resets to 0. */
@@ -165,6 +167,20 @@ int sparse_mla_decode_num_splits(int batch, int n_heads, int topk, int config);
 
 /* Bytes of workspace sparse_mla_decode_launcher needs for these sizes and this config. */
 size_t sparse_mla_decode_workspace_bytes(int batch, int n_heads, int topk, int config);
+
+/* sparse_mla_decode_launcher without a workspace argument. No counterpart in the reference workspace: it is for
+ * callers that cannot allocate device memory (code under HIP graph capture, serving loops with a fixed memory
+ * plan, harnesses that forbid hipMalloc). The partial outputs of the key splits go to a static device array of
+ * the library (sparse_mla_decode_static_scratch_bytes() = 72 MiB per GPU, held from module load to process end);
+ * the kernels and the result are those of sparse_mla_decode_launcher, bit for bit. A problem whose
+ * sparse_mla_decode_workspace_bytes(...) exceeds that size is rejected (status 4) and nothing is launched.
+ * All calls on one GPU share the array: calls that overlap in time on one GPU race, calls on one stream are safe.
+ * The first call on a device looks up the array's address and must not be made under graph capture; no call
+ * allocates or frees memory. */
+size_t sparse_mla_decode_static_scratch_bytes(void);
+void sparse_mla_decode_static_launcher(void* out, const void* q, const void* kv, const int* idx, int batch,
+                                       int n_heads, int n_kv_rows, int topk, int d_qk, int d_v,
+                                       float sm_scale, int out_dtype, int config, hipStream_t stream);
 
 /* e4m3 storage form of the latent cache (caller-side neighbour of sparse_mla_decode_launcher; same launcher
  * pattern agent_workdir/kernels/axpby.cu:12-20). A row is 656 bytes: 512 e4m3 codes of the latent values,
