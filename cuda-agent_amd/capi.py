@@ -74,6 +74,7 @@ SIGNATURES = {
                                              c_int, c_int, c_int, c_int, _P]),
     'moe_fp8_workspace_bytes': (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
     'moe_fp8_workspace_layout': (None, [_P, c_int, c_int, c_int, c_int, c_int]),
+    'moe_fp8_uses_tiled_gemms': (c_int, [c_int, c_int, c_int, c_int, c_int, c_int]),
     'moe_fp8_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int,
                                 c_int, c_int, c_int, _P]),
 }
@@ -521,7 +522,7 @@ def topk_select_launch(idx_out, scores, lengths=None, stream=None):
 
 
 MOE_WORKSPACE_FIELDS = ('ids', 'weights', 'expert_offsets', 'sorted_pairs', 'pair_pos', 'x_q', 'x_s',
-                        'h_q', 'h_s', 'y', 'h_marks')
+                        'h_q', 'h_s', 'y', 'h_marks', 'y_scale')
 
 
 def moe_workspace_bytes(tokens, hidden, inter, n_experts, top_k=8):
@@ -540,7 +541,7 @@ def moe_workspace_views(workspace, tokens, hidden, inter, n_experts, top_k=8):
         'pair_pos': (torch.int32, (pairs,)), 'x_q': (torch.float8_e4m3fn, (tokens, hidden)),
         'x_s': (torch.float32, (tokens, hidden // 128)), 'h_q': (torch.float8_e4m3fn, (pairs, inter)),
         'h_s': (torch.float32, (pairs, inter // 128)), 'y': (torch.float32, (pairs, hidden)),
-        'h_marks': (torch.uint8, (pairs, inter)),
+        'h_marks': (torch.uint8, (pairs, inter)), 'y_scale': (torch.float32, (pairs, (hidden + 255) // 256)),
     }
     views = {}
     for name, off in zip(MOE_WORKSPACE_FIELDS, offs):
@@ -551,6 +552,19 @@ def moe_workspace_views(workspace, tokens, hidden, inter, n_experts, top_k=8):
         nbytes = n * torch.empty((), dtype=dtype).element_size()
         views[name] = workspace[off:off + nbytes].view(dtype).view(shape)
     return views
+
+
+def moe_expert_outputs(views, tokens, hidden, inter, n_experts, top_k=8, config=0):
+    """The expert outputs y [tokens*top_k, hidden] of a finished layer as fp32, whichever way the layer stored
+    them: fp32 rows (weight-streaming GEMMs) or fp16 rows with power-of-two scales (LDS-tiled GEMMs)."""
+    import torch
+    tiled = library().moe_fp8_uses_tiled_gemms(tokens, hidden, inter, n_experts, top_k, config)
+    _require(tiled >= 0, 'moe_expert_outputs: unsupported shape')
+    if not tiled:
+        return views['y']
+    pairs = tokens * top_k
+    half = views['y'].reshape(-1).view(torch.float16)[:pairs * hidden].view(pairs, hidden)
+    return half.float() * views['y_scale'].repeat_interleave(256, dim=1)
 
 
 def moe_route_launch(ids, weights, logits, stream=None):

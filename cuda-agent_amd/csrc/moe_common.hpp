@@ -109,7 +109,9 @@ struct Workspace {
     float* x_s;           // [T*H/128]
     uint8_t* h_q;         // [T*k*I] e4m3 silu(g)*u, rows in sorted order
     float* h_s;           // [T*k*I/128]
-    float* y;             // [T*k*H] expert outputs, rows in sorted order
+    float* y;             // [T*k*H] expert outputs, rows in sorted order: fp32 from the streaming down GEMM; from
+                          //         the tiled one fp16 of y / y_scale in the first half of the buffer
+    float* y_scale;       // [T*k][H/256] power of two above the largest |y| of each run of 256 columns (tiled)
     int* tile_start;      // [E+1]  first 256-pair tile of every expert (tiled path)
     float* xs_t;          // [H/128][scale_stride] activation scales by sorted position, transposed
     float* hs_t;          // [I/128][scale_stride] the same for h
@@ -148,6 +150,7 @@ inline Workspace carve_workspace(void* base, int tokens, int hidden, int inter, 
     w.xs_t = reinterpret_cast<float*>(take((size_t)(hidden / GROUP) * w.scale_stride * 4));
     w.hs_t = reinterpret_cast<float*>(take((size_t)(inter / GROUP) * w.scale_stride * 4));
     w.h_marks = reinterpret_cast<uint8_t*>(take(pairs * inter));
+    w.y_scale = reinterpret_cast<float*>(take(pairs * ((hidden + 255) / 256) * 4));
     w.bytes = off;
     return w;
 }

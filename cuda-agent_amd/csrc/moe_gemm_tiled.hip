@@ -121,6 +121,8 @@ __global__ __launch_bounds__(256) void moe_gather_scales_kernel(const float* __r
 // cycles it spends in each phase of the K loop and leaves them in g_phase_cycles.
 #ifdef MOE_PHASE_TIMING
 __device__ unsigned long long g_phase_cycles[8][8];
+// and every workgroup leaves its start and end on the 100 MHz wall clock, its pair count and its hardware id
+__device__ unsigned long long g_wg_trace[16384][3];
 #define PHASE_TIMING_BEGIN()                                                              \
     unsigned long long phase_t0 = __builtin_readcyclecounter(), phase_acc[8] = {};        \
     const unsigned long long phase_wall0 = wall_clock64(), phase_core0 = phase_t0
@@ -135,6 +137,11 @@ __device__ unsigned long long g_phase_cycles[8][8];
         for (int i = 0; i < 7; ++i) g_phase_cycles[wave][i] = phase_acc[i]; \
         /* core clock in kHz over the workgroup's life: the wall clock counts at 100 MHz */ \
         g_phase_cycles[wave][7] = (__builtin_readcyclecounter() - phase_core0) * 100000ull / (wall_clock64() - phase_wall0); \
+    }                                                                       \
+    if ((wave) == 0 && (lane) == 0 && blockIdx.x < 16384) {                 \
+        g_wg_trace[blockIdx.x][0] = phase_wall0;                            \
+        g_wg_trace[blockIdx.x][1] = wall_clock64();                         \
+        g_wg_trace[blockIdx.x][2] = ((unsigned long long)cnt << 32) | __builtin_amdgcn_s_getreg((31 << 11) | 4); \
     }
 #else
 #define PHASE_TIMING_BEGIN()
@@ -154,8 +161,8 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
     const float* __restrict__ as_t, const int* __restrict__ sorted_pairs,
     const int* __restrict__ expert_offsets, const int* __restrict__ tile_start,
     uint8_t* __restrict__ h_q, float* __restrict__ h_s, float* __restrict__ hs_t, float* __restrict__ y,
-    int K, int n_rows, int inter, int top_k, int n_experts, int scale_stride,
-    uint8_t* __restrict__ h_marks = nullptr, float err_coef = 0.f) {
+    float* __restrict__ y_scale, int K, int n_rows, int inter, int top_k, int n_experts, int scale_stride,
+    uint8_t* __restrict__ h_marks, float err_coef) {
     __shared__ __attribute__((aligned(16))) uint8_t s_stage[2 * STAGE_BYTES];
 
     // Workgroup -> (row tile, pair tile). Consecutive workgroup ids go round-robin to the 8 XCDs,
@@ -572,37 +579,65 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
             }
         }
     } else {
-        // two passes of 128 pairs: the wavefronts of one pair half put their 64 x 128 results into
-        // LDS as [pair][256 rows], then all 8 wavefronts write whole 1 KB rows
-        constexpr int Y_ROW = TILE_ROWS + 4;  // floats per staged pair row (16 bytes of padding)
-        static_assert(128 * Y_ROW * sizeof(float) <= 2 * STAGE_BYTES, "epilogue LDS");
-        float* s_y = reinterpret_cast<float*>(s_stage);
+        // The tile leaves as fp16 of y / 2^e, 2^e the power of two above the largest magnitude of the pair's 256
+        // values of this tile (kept per pair and column tile for the combine): half the bytes of fp32 to write
+        // here and to read there, 11 significant bits relative to that maximum. The maximum of a pair: over a
+        // lane's 32 values, the lane holding the pair's other rows of this wavefront, and through LDS the four
+        // wavefronts that hold its other row groups. Then two passes of 128 pairs: the wavefronts of one pair
+        // half put their 64 x 128 results into LDS as [pair][256 rows], and all 8 wavefronts write whole
+        // 512-byte rows.
+        typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
+        constexpr int Y_ROW = TILE_ROWS + 8;  // halfs per staged pair row (16 bytes of padding)
+        _Float16* s_y = reinterpret_cast<_Float16*>(s_stage);
+        float* s_max = reinterpret_cast<float*>(s_stage + 128 * Y_ROW * sizeof(_Float16));  // [4 row groups][256 pairs]
+        static_assert(128 * Y_ROW * sizeof(_Float16) + 4 * TILE_PAIRS * sizeof(float) <= 2 * STAGE_BYTES, "epilogue LDS");
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            float m = 0.f;
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) m = fmaxf(m, fabsf(acc[a][b][i]));
+            m = fmaxf(m, __shfl_xor(m, 32));
+            if (half == 0) s_max[rg * TILE_PAIRS + th * 128 + b * 32 + r32] = m;
+        }
+        __syncthreads();
+        auto pair_exponent = [&](int pl) {  // biased exponent of 2^e for pair pl of the tile
+            const float m = fmaxf(fmaxf(s_max[pl], s_max[TILE_PAIRS + pl]),
+                                  fmaxf(s_max[2 * TILE_PAIRS + pl], s_max[3 * TILE_PAIRS + pl]));
+            const uint32_t e_bits = ((__float_as_uint(m) >> 23) & 255u) + 1u;
+            return m > 0.f ? (e_bits > 253u ? 253u : e_bits) : 127u;
+        };
 #pragma unroll
         for (int pass = 0; pass < 2; ++pass) {
             if (pass == 1) __syncthreads();
             if (th == pass) {
 #pragma unroll
                 for (int b = 0; b < 4; ++b) {
-                    float* dst = s_y + (b * 32 + r32) * Y_ROW + rg * 64 + 4 * half;
+                    const float inv = __uint_as_float((254u - pair_exponent(th * 128 + b * 32 + r32)) << 23);
+                    _Float16* dst = s_y + (b * 32 + r32) * Y_ROW + rg * 64 + 4 * half;
 #pragma unroll
                     for (int a = 0; a < 2; ++a) {
 #pragma unroll
                         for (int qd = 0; qd < 4; ++qd) {
-                            *reinterpret_cast<floatx4*>(dst + a * 32 + 8 * qd) =
-                                floatx4{acc[a][b][4 * qd], acc[a][b][4 * qd + 1], acc[a][b][4 * qd + 2],
-                                        acc[a][b][4 * qd + 3]};
+                            *reinterpret_cast<halfx4*>(dst + a * 32 + 8 * qd) =
+                                halfx4{(_Float16)(acc[a][b][4 * qd] * inv), (_Float16)(acc[a][b][4 * qd + 1] * inv),
+                                       (_Float16)(acc[a][b][4 * qd + 2] * inv), (_Float16)(acc[a][b][4 * qd + 3] * inv)};
                         }
                     }
                 }
             }
             __syncthreads();
+            // 32 lanes write the 512 bytes of one pair: two pairs per instruction, 8 instructions per wavefront
 #pragma unroll
-            for (int it = 0; it < 16; ++it) {
-                const int pr = wave * 16 + it;  // pair within this half
+            for (int it = 0; it < 8; ++it) {
+                const int pr = wave * 16 + 2 * it + half;  // pair within this half
                 const int pl = pass * 128 + pr;
                 if (pl < cnt) {
-                    const floatx4 v = *reinterpret_cast<const floatx4*>(s_y + pr * Y_ROW + lane * 4);
-                    *reinterpret_cast<floatx4*>(y + ((size_t)begin + pl) * n_rows + rb * TILE_ROWS + lane * 4) = v;
+                    const size_t row = (size_t)begin + pl;
+                    *reinterpret_cast<intx4*>(reinterpret_cast<_Float16*>(y) + row * n_rows + rb * TILE_ROWS + r32 * 8) =
+                        *reinterpret_cast<const intx4*>(s_y + pr * Y_ROW + r32 * 8);
+                    if (r32 == 0) y_scale[row * (n_rows / TILE_ROWS) + rb] = __uint_as_float(pair_exponent(pl) << 23);
                 }
             }
         }
@@ -652,7 +687,7 @@ extern "C" void moe_gate_up_tiled_marked_launcher(void* h_q, float* h_s, float* 
                                 : (ue8m0 ? moe_tiled_gemm_kernel<true, true, false> : moe_tiled_gemm_kernel<true, false, false>);
     kernel<<<grid, 512, 0, stream>>>(
         static_cast<const uint8_t*>(w13_q), w13_s, static_cast<const uint8_t*>(x_q), xs_t, sorted_pairs,
-        expert_offsets, tile_start, static_cast<uint8_t*>(h_q), h_s, hs_t, nullptr, hidden, 2 * inter,
+        expert_offsets, tile_start, static_cast<uint8_t*>(h_q), h_s, hs_t, nullptr, nullptr, hidden, 2 * inter,
         inter, top_k, n_experts, scale_stride, static_cast<uint8_t*>(h_marks),
         requant_error_coefficient(band_config));
 }
@@ -668,8 +703,10 @@ extern "C" void moe_gate_up_tiled_launcher(void* h_q, float* h_s, float* hs_t, c
                                       scale_stride, ue8m0, 0, stream);
 }
 
-extern "C" void moe_down_tiled_launcher(float* y, const void* h_q, const float* hs_t, const void* w2_q,
-                                        const float* w2_s, const int* expert_offsets,
+// y [pairs, hidden] as fp16 of y / y_scale (the buffer's first pairs * hidden * 2 bytes), y_scale
+// [pairs, hidden/256] fp32 powers of two: value = fp16 * y_scale[row][column / 256].
+extern "C" void moe_down_tiled_launcher(void* y, float* y_scale, const void* h_q, const float* hs_t,
+                                        const void* w2_q, const float* w2_s, const int* expert_offsets,
                                         const int* tile_start, int tokens, int hidden, int inter,
                                         int n_experts, int top_k, int scale_stride, int ue8m0,
                                         hipStream_t stream) {
@@ -684,6 +721,6 @@ extern "C" void moe_down_tiled_launcher(float* y, const void* h_q, const float* 
     const auto kernel = ue8m0 ? moe_tiled_gemm_kernel<false, true> : moe_tiled_gemm_kernel<false, false>;
     kernel<<<grid, 512, 0, stream>>>(
         static_cast<const uint8_t*>(w2_q), w2_s, static_cast<const uint8_t*>(h_q), hs_t, nullptr,
-        expert_offsets, tile_start, nullptr, nullptr, nullptr, y, inter, hidden, inter, top_k,
-        n_experts, scale_stride, nullptr, 0.f);
+        expert_offsets, tile_start, nullptr, nullptr, nullptr, static_cast<float*>(y), y_scale, inter, hidden,
+        inter, top_k, n_experts, scale_stride, nullptr, 0.f);
 }

@@ -47,8 +47,8 @@ extern "C" void moe_gate_up_tiled_launcher(void* h_q, float* h_s, float* hs_t, c
                                            const int* tile_start, int tokens, int hidden, int inter,
                                            int n_experts, int top_k, int scale_stride, int ue8m0,
                                            hipStream_t stream);
-extern "C" void moe_down_tiled_launcher(float* y, const void* h_q, const float* hs_t, const void* w2_q,
-                                        const float* w2_s, const int* expert_offsets,
+extern "C" void moe_down_tiled_launcher(void* y, float* y_scale, const void* h_q, const float* hs_t,
+                                        const void* w2_q, const float* w2_s, const int* expert_offsets,
                                         const int* tile_start, int tokens, int hidden, int inter,
                                         int n_experts, int top_k, int scale_stride, int ue8m0,
                                         hipStream_t stream);
@@ -73,13 +73,32 @@ __global__ __launch_bounds__(256) void moe_identity_sort_kernel(int* __restrict_
     if (i < 2) expert_offsets[i] = i * tokens;
 }
 
+typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
+
+// Four consecutive values of row `row` of an expert-output buffer at column c: fp32 rows, or (HALF) fp16 rows
+// with one power-of-two scale per row and run of 256 columns, as the tiled down GEMM stores them.
+template <bool HALF>
+__device__ __forceinline__ floatx4 load_y4(const void* y, const float* y_scale, size_t row, int hidden, int c) {
+    if constexpr (HALF) {
+        const halfx4 v = __builtin_nontemporal_load(
+            reinterpret_cast<const halfx4*>(static_cast<const _Float16*>(y) + row * hidden + c));
+        const float s = y_scale[row * (size_t)(hidden / 256) + (c >> 8)];
+        return floatx4{(float)v.x * s, (float)v.y * s, (float)v.z * s, (float)v.w * s};
+    } else {
+        return __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(static_cast<const float*>(y) + row * hidden + c));
+    }
+}
+
 // out[t, :] = sum_k weights[t, k] * y[pair_pos[t*top_k + k], :] (k ascending) + y_shared[t, :], fp32.
 // blockIdx.x is the token, blockIdx.y a 1024-column slice; 4 columns per lane.
-template <typename OUT>
-__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y,
+// YH / SH: the routed / the shared expert outputs are in the fp16 form (see load_y4).
+template <typename OUT, bool YH, bool SH>
+__global__ __launch_bounds__(256) void moe_combine_kernel(const void* __restrict__ y,
+                                                          const float* __restrict__ y_scale,
                                                           const float* __restrict__ weights,
                                                           const int* __restrict__ pair_pos,
-                                                          const float* __restrict__ y_shared,
+                                                          const void* __restrict__ y_shared,
+                                                          const float* __restrict__ ys_scale,
                                                           OUT* __restrict__ out, int hidden,
                                                           int top_k) {
     const int t = blockIdx.x;
@@ -94,7 +113,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
                 const int k = k0 + j < top_k ? k0 + j : k0;
                 const int pos = pair_pos[(size_t)t * top_k + k];
                 w[j] = weights[(size_t)t * top_k + k];
-                v[j] = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(y + (size_t)pos * hidden + c));
+                v[j] = load_y4<YH>(y, y_scale, (size_t)pos, hidden, c);
             }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -102,8 +121,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
             }
         }
         // the shared expert's row, if there is one, is added last
-        if (y_shared != nullptr)
-            acc += __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(y_shared + (size_t)t * hidden + c));
+        if (y_shared != nullptr) acc += load_y4<SH>(y_shared, ys_scale, (size_t)t, hidden, c);
         OUT* dst = out + (size_t)t * hidden + c;
         if constexpr (sizeof(OUT) == 4) {
             *reinterpret_cast<floatx4*>(dst) = acc;
@@ -112,6 +130,28 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
             *reinterpret_cast<bf16x4*>(dst) = r;
         }
     }
+}
+
+// y_scale / ys_scale null: that buffer holds fp32 rows; else the fp16 form with these scales (hidden % 256 == 0)
+void launch_combine(void* out, const void* y, const float* y_scale, const float* weights, const int* pair_pos,
+                    const void* y_shared, const float* ys_scale, int tokens, int hidden, int top_k, int out_dtype,
+                    hipStream_t stream) {
+    const dim3 grid(tokens, (hidden + 1023) / 1024);
+#define MOE_COMBINE(OUT_T, YH, SH)                                                                              \
+    moe_combine_kernel<OUT_T, YH, SH><<<grid, 256, 0, stream>>>(y, y_scale, weights, pair_pos, y_shared, ys_scale, \
+                                                               static_cast<OUT_T*>(out), hidden, top_k)
+#define MOE_COMBINE_FORMS(OUT_T)                             \
+    if (y_scale && ys_scale) MOE_COMBINE(OUT_T, true, true); \
+    else if (y_scale) MOE_COMBINE(OUT_T, true, false);       \
+    else if (ys_scale) MOE_COMBINE(OUT_T, false, true);      \
+    else MOE_COMBINE(OUT_T, false, false)
+    if (out_dtype == 0) {
+        MOE_COMBINE_FORMS(__bf16);
+    } else {
+        MOE_COMBINE_FORMS(float);
+    }
+#undef MOE_COMBINE_FORMS
+#undef MOE_COMBINE
 }
 
 }  // namespace
@@ -134,14 +174,7 @@ extern "C" void moe_combine_shared_launcher(void* out, const float* y, const flo
         caa::set_status(CAA_BAD_ARGUMENT);
         return;
     }
-    const dim3 grid(tokens, (hidden + 1023) / 1024);
-    if (out_dtype == 0) {
-        moe_combine_kernel<__bf16><<<grid, 256, 0, stream>>>(y, weights, pair_pos, y_shared,
-                                                            static_cast<__bf16*>(out), hidden, top_k);
-    } else {
-        moe_combine_kernel<float><<<grid, 256, 0, stream>>>(y, weights, pair_pos, y_shared,
-                                                           static_cast<float*>(out), hidden, top_k);
-    }
+    launch_combine(out, y, nullptr, weights, pair_pos, y_shared, nullptr, tokens, hidden, top_k, out_dtype, stream);
 }
 
 extern "C" void moe_combine_launcher(void* out, const float* y, const float* weights,
@@ -158,15 +191,15 @@ extern "C" size_t moe_fp8_workspace_bytes(int tokens, int hidden, int inter, int
 }
 
 // Byte offsets of the intermediate buffers inside the workspace, in the order
-// ids, weights, expert_offsets, sorted_pairs, pair_pos, x_q, x_s, h_q, h_s, y, h_marks
+// ids, weights, expert_offsets, sorted_pairs, pair_pos, x_q, x_s, h_q, h_s, y, h_marks, y_scale
 // (for checkers that compare the stages against a reference).
-extern "C" void moe_fp8_workspace_layout(size_t* offsets11, int tokens, int hidden, int inter,
+extern "C" void moe_fp8_workspace_layout(size_t* offsets12, int tokens, int hidden, int inter,
                                          int n_experts, int top_k) {
     char* base = reinterpret_cast<char*>(uintptr_t{4096});
     const moe::Workspace w = moe::carve_workspace(base, tokens, hidden, inter, n_experts, top_k);
-    const void* ptrs[11] = {w.ids, w.weights, w.expert_offsets, w.sorted_pairs, w.pair_pos, w.x_q,
-                            w.x_s, w.h_q,     w.h_s,            w.y,            w.h_marks};
-    for (int i = 0; i < 11; ++i) offsets11[i] = static_cast<const char*>(ptrs[i]) - base;
+    const void* ptrs[12] = {w.ids, w.weights, w.expert_offsets, w.sorted_pairs, w.pair_pos, w.x_q,
+                            w.x_s, w.h_q,     w.h_s,            w.y,            w.h_marks,  w.y_scale};
+    for (int i = 0; i < 12; ++i) offsets12[i] = static_cast<const char*>(ptrs[i]) - base;
 }
 
 namespace {
@@ -218,7 +251,7 @@ void run_expert_gemms(const moe::Workspace& w, const GemmPlan& plan, const void*
             moe_requant_fix_launcher(w.h_q, w.h_s, w.hs_t, marks, w.x_q, w.x_s, w13_q, w13_s, w.sorted_pairs,
                                      w.expert_offsets, tokens, hidden, inter, n_experts, top_k, w.scale_stride,
                                      ue8m0, stream);
-        moe_down_tiled_launcher(w.y, w.h_q, w.hs_t, w2_q, w2_s, w.expert_offsets, w.tile_start, tokens,
+        moe_down_tiled_launcher(w.y, w.y_scale, w.h_q, w.hs_t, w2_q, w2_s, w.expert_offsets, w.tile_start, tokens,
                                 hidden, inter, n_experts, top_k, w.scale_stride, ue8m0, stream);
     } else {
         moe_gate_up_launcher(w.h_q, w.h_s, w.x_q, w.x_s, w13_q, w13_s, w.sorted_pairs, w.expert_offsets,
@@ -235,6 +268,14 @@ bool layer_shape_ok(int hidden, int inter, int n_experts, int top_k, int tokens,
 }
 
 }  // namespace
+
+// 1 if moe_fp8_launcher runs these sizes and this config on the LDS-tiled GEMMs, 0 if on the weight-streaming
+// ones (for checkers: the form decides how the workspace's y buffer is laid out), -1 for an unsupported shape.
+extern "C" int moe_fp8_uses_tiled_gemms(int tokens, int hidden, int inter, int n_experts, int top_k, int config) {
+    if (tokens <= 0 || !layer_shape_ok(hidden, inter, n_experts, top_k, tokens, 0)) return -1;
+    const GemmPlan plan = plan_expert_gemms(tokens, hidden, inter, n_experts, top_k, config);
+    return plan.ok ? (plan.tiled ? 1 : 0) : -1;
+}
 
 // The whole layer. out [tokens, hidden] bf16 (out_dtype 0) or fp32 (out_dtype 1).
 // config: 0 = choose by the average number of pairs per expert (above 32: LDS-tiled GEMMs, else
@@ -269,7 +310,8 @@ extern "C" void moe_fp8_launcher(void* out, const void* x, const float* logits, 
                             logits, tokens, n_experts, top_k, 0, stream);
     moe_quant_bf16_launcher(w.x_q, w.x_s, x, tokens, hidden, config & CONFIG_UE8M0, stream);
     run_expert_gemms(w, plan, w13_q, w13_s, w2_q, w2_s, tokens, hidden, inter, n_experts, top_k, config, stream);
-    moe_combine_launcher(out, w.y, w.weights, w.pair_pos, tokens, hidden, top_k, out_dtype, 0, stream);
+    launch_combine(out, w.y, plan.tiled ? w.y_scale : nullptr, w.weights, w.pair_pos, nullptr, nullptr, tokens, hidden,
+                   top_k, out_dtype, stream);
 }
 
 // Workspace of moe_fp8_shared_launcher: the routed experts' workspace followed by the same
@@ -325,8 +367,8 @@ extern "C" void moe_fp8_shared_launcher(void* out, const void* x, const float* l
                                                                       sh.expert_offsets, tokens);
     run_expert_gemms(sh, shared_plan, sw13_q, sw13_s, sw2_q, sw2_s, tokens, hidden, shared_inter, 1, 1, config,
                      stream);
-    moe_combine_shared_launcher(out, w.y, w.weights, w.pair_pos, sh.y, tokens, hidden, top_k, out_dtype,
-                                0, stream);
+    launch_combine(out, w.y, plan.tiled ? w.y_scale : nullptr, w.weights, w.pair_pos, sh.y,
+                   shared_plan.tiled ? sh.y_scale : nullptr, tokens, hidden, top_k, out_dtype, stream);
 }
 
 // The layer with a shared expert stored as expert number n_experts behind the routed ones
@@ -364,6 +406,7 @@ extern "C" void moe_fp8_fused_shared_launcher(void* out, const void* x, const fl
     moe_quant_bf16_launcher(w.x_q, w.x_s, x, tokens, hidden, config & CONFIG_UE8M0, stream);
     run_expert_gemms(w, plan, w13_q, w13_s, w2_q, w2_s, tokens, hidden, inter, n_experts + 1, top_k + 1,
                      (config & ~CONFIG_LAST_EXPERT_FIRST) | CONFIG_LAST_EXPERT_FIRST, stream);
-    moe_combine_launcher(out, w.y, w.weights, w.pair_pos, tokens, hidden, top_k + 1, out_dtype, 0, stream);
+    launch_combine(out, w.y, plan.tiled ? w.y_scale : nullptr, w.weights, w.pair_pos, nullptr, nullptr, tokens, hidden,
+                   top_k + 1, out_dtype, stream);
 }
 

@@ -382,12 +382,19 @@ void moe_combine_launcher(void* out, const float* y, const float* weights, const
 size_t moe_fp8_workspace_bytes(int tokens, int hidden, int inter, int n_experts, int top_k);
 
 /* Byte offsets, inside that workspace, of ids, weights, expert_offsets, sorted_pairs, pair_pos,
- * x_q, x_s, h_q, h_s, y, h_marks (in this order), for checkers that inspect the stages. h_marks
- * [tokens*top_k, inter] bytes: bit 0 = the element was within the matrix core's error of an e4m3
- * rounding boundary, bit 1 = it may have been its group's maximum (written only when the exact
+ * x_q, x_s, h_q, h_s, y, h_marks, y_scale (in this order), for checkers that inspect the stages.
+ * y [tokens*top_k, hidden]: fp32 rows when the layer ran the weight-streaming GEMMs; when it ran the
+ * LDS-tiled ones (moe_fp8_uses_tiled_gemms), fp16 rows in the first half of the buffer, to be
+ * multiplied by y_scale [tokens*top_k, hidden/256] (one power of two per row and run of 256 columns).
+ * h_marks [tokens*top_k, inter] bytes: bit 0 = the element was within the matrix core's error of an
+ * e4m3 rounding boundary, bit 1 = it may have been its group's maximum (written only when the exact
  * requantisation pass runs, see moe_fp8_launcher). */
-void moe_fp8_workspace_layout(size_t* offsets11, int tokens, int hidden, int inter, int n_experts,
+void moe_fp8_workspace_layout(size_t* offsets12, int tokens, int hidden, int inter, int n_experts,
                               int top_k);
+
+/* 1 if moe_fp8_launcher runs these sizes and this config on the LDS-tiled GEMMs, 0 if on the
+ * weight-streaming ones, -1 if it rejects them. */
+int moe_fp8_uses_tiled_gemms(int tokens, int hidden, int inter, int n_experts, int top_k, int config);
 
 /* The whole layer: out [tokens, hidden] (bf16 if out_dtype == 0, the operator's output type;
  * fp32 if 1, the same values before the final rounding) from x [tokens, hidden] bf16 and

@@ -40,7 +40,10 @@ def run_layer(capi, dev_tensors, top_k, config=0, dtype=torch.bfloat16):
     out = torch.full((T, H), float('nan'), dtype=dtype, device=x.device)
     capi.moe_fp8_launch(out, x, logits, w13_q, w13_s, w2_q, w2_s, ws, top_k=top_k, config=config)
     torch.cuda.synchronize()
-    return out, capi.moe_workspace_views(ws, T, H, I2 // 2, E, top_k)
+    views = capi.moe_workspace_views(ws, T, H, I2 // 2, E, top_k)
+    # the expert outputs as fp32, whichever way this form of the layer stores them
+    views['y'] = capi.moe_expert_outputs(views, T, H, I2 // 2, E, top_k, config)
+    return out, views
 
 
 @pytest.mark.parametrize('shape', [(64, 256, 8), (1000, 64, 6), (5, 512, 8), (700, 256, 8)])
@@ -131,9 +134,10 @@ def check_layer(capi, dev, T, H, I, E, k, seed, config=0, biased=None):
     code_diff = code_steps(hq, mid['h_q'])
     assert (code_diff > 0).float().mean().item() < 2e-4
     assert not (code_diff > 1).any()                         # never more than one code step
-    # down projection, on the kernel's own h
+    # down projection, on the kernel's own h (the tiled form stores y with 11 significant bits relative to the
+    # largest value of each run of 256 columns: up to 2.5e-3 of the rms)
     y = views['y'].cpu()[pos].reshape(T, k, H)
-    assert moe.rel_rms_error(y, oracle_down(hq, hs, mid['ids'], w2_q, w2_s)) <= 1e-3
+    assert moe.rel_rms_error(y, oracle_down(hq, hs, mid['ids'], w2_q, w2_s)) <= 3e-3
     # combine, on the kernel's own y
     want = torch.zeros(T, H)
     for j in range(k):
@@ -375,7 +379,7 @@ def check_sampled_tokens(tokens, dts, ids, pos, views, exact, k, exact_requant=T
     assert not far.any() if exact_requant else far.float().mean().item() < 1e-4
     y = views['y'][rows].cpu().reshape(n, k, H)
     local = dict(mid, ids=mid['local_ids'])
-    assert moe.rel_rms_error(y, oracle_down(hq, hs, mid['local_ids'], w2_q, w2_s)) <= 1e-3
+    assert moe.rel_rms_error(y, oracle_down(hq, hs, mid['local_ids'], w2_q, w2_s)) <= 3e-3
     want = torch.zeros(n, H)
     for j in range(k):
         want += mid['weights'][:, j:j + 1] * y[:, j]

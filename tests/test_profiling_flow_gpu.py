@@ -1,0 +1,87 @@
+"""The workspace's timing flow (`python3 -m utils.profiling`, the counterpart of
+agent_workdir/utils/profiling.py:59-117) on the GPU for the three operators: the result line has the
+reference's format, the figure of the extension comes from the profiler's device-time sum (not from the
+HIP-event fallback), it does not exceed the stream time measured by events around the same loop, and for the
+two operators that are one or two long kernels it agrees within 10 % with the event time of the same launch
+through the C ABI, which is how bench.py times it."""
+import os
+import re
+import subprocess
+import sys
+from pathlib import Path
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+WORKSPACES = Path(__file__).resolve().parent.parent / 'cuda-agent_amd' / 'workspaces'
+RESULT_LINE = re.compile(r'^Torch Baseline: (\d+\.\d{3})us, Torch Compile: (\d+\.\d{3})us, CUDA Extension: (\d+\.\d{3})us$',
+                         re.M)
+TIMING_LINE = re.compile(r'^\[timing\] cuda_extension: profiler device time, (\d+) GPU events '
+                         r'\(stream time by events (\d+\.\d{3})us\)$', re.M)
+
+
+def run_flow(workspace, env):
+    ws = WORKSPACES / workspace
+    assert (ws / 'cuda_extension.so').exists(), 'workspace extension not built'
+    out = subprocess.run([sys.executable, '-m', 'utils.profiling', '--iters', '3'], cwd=ws,
+                         env=dict(os.environ, **env), capture_output=True, text=True, timeout=900)
+    assert out.returncode == 0, out.stdout + out.stderr
+    result = RESULT_LINE.search(out.stdout)
+    assert result, out.stdout
+    timing = TIMING_LINE.search(out.stdout)
+    assert timing, 'the extension was not timed by the profiler:\n' + out.stdout
+    eager_us, compiled_us, ext_us = (float(v) for v in result.groups())
+    n_events, stream_us = int(timing.group(1)), float(timing.group(2))
+    print(f'[profiling] {workspace} {env}: eager {eager_us:.1f} us, torch.compile {compiled_us:.1f} us, '
+          f'extension {ext_us:.1f} us ({n_events} GPU events in 3 forwards, {stream_us:.1f} us of stream time each)')
+    assert n_events >= 3 and 0 < ext_us <= stream_us * 1.02
+    return eager_us, compiled_us, ext_us
+
+
+def event_time_us(launch, warmup=5, iters=10):
+    for _ in range(warmup):
+        launch()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        launch()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) * 1e3 / iters
+
+
+def test_gdn_decode_workload(capi, dev):
+    _, compiled_us, ext_us = run_flow('gdn_decode', {'GDN_CONFIG': '1'})
+    B, Hv, Hqk = 256, 32, 16
+    q = torch.randn(B, Hqk, 128, device=dev).bfloat16()
+    k = torch.randn(B, Hqk, 128, device=dev).bfloat16()
+    v = torch.randn(B, Hv, 128, device=dev).bfloat16()
+    g = torch.rand(B, Hv, device=dev)
+    beta = torch.rand(B, Hv, device=dev)
+    state = 0.02 * torch.randn(B, Hv, 128, 128, device=dev)
+    o = torch.empty(B, Hv, 128, device=dev)
+    mine = event_time_us(lambda: capi.gdn_decode_launch(o, state, q, k, v, g, beta))
+    assert abs(ext_us - mine) <= 0.10 * mine, (ext_us, mine)
+    assert ext_us <= 0.95 * compiled_us        # the workspace's pass bar against torch.compile
+
+
+def test_sparse_mla_workload(capi, dev):
+    _, compiled_us, ext_us = run_flow('sparse_mla', {'MLA_CONFIG': '3'})
+    B, H, N, topk = 64, 128, 32768, 2048
+    q = torch.randn(B, H, 576, device=dev).bfloat16()
+    kv = torch.randn(B, N, 576, device=dev).bfloat16()
+    idx = torch.stack([torch.randperm(N, device=dev)[:topk] for _ in range(B)]).int()
+    out = torch.empty(B, H, 512, dtype=torch.bfloat16, device=dev)
+    ws = torch.empty(capi.sparse_mla_workspace_bytes(B, H, topk), dtype=torch.uint8, device=dev)
+    mine = event_time_us(lambda: capi.sparse_mla_decode_launch(out, q, kv, idx, ws))
+    assert abs(ext_us - mine) <= 0.10 * mine, (ext_us, mine)
+    assert ext_us <= 0.95 * compiled_us
+
+
+def test_moe_reduced_layer():
+    # (a chain of ten short kernels: their device times add up to about half the stream time, so only the
+    # format, the timing source and the pass bar are checked)
+    _, compiled_us, ext_us = run_flow('moe_fp8', {'MOE_CONFIG': 'small'})
+    assert ext_us <= 0.95 * compiled_us
