@@ -542,7 +542,7 @@ def moe_cpu_baseline(torch, tensors, n_tokens):
     return csec, len(used), cores
 
 
-def bench_moe(torch, capi, dev, steps, warmup, cpu_baseline, prefill):
+def bench_moe(torch, capi, dev, steps, warmup, cpu_baseline, prefill, plain=False):
     T = 8192 if prefill else 64
     H, I, E, k = 7168, 2048, 256, 8
     tensors, stacked = make_moe(torch, dev, T, prefill)
@@ -573,6 +573,8 @@ def bench_moe(torch, capi, dev, steps, warmup, cpu_baseline, prefill):
             roofline=dict(bound="hbm", achieved=wbytes / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
                           frac=wbytes / sec / 1e9 / HBM_PEAK_GBS, traffic=MEASURED_TRAFFIC['moe_decode']),
             algorithmic_bytes=wbytes, active_experts=n_active, tflops=flops / sec / 1e12)
+    if plain:  # (the workload's own kernels only: what a profiler run wants)
+        return res
     # the same layer with a shared expert (one more block-scaled MLP of inter 2048 on every token): as launches
     # of its own, and stored behind the routed experts so that it runs inside their launches
     sw13_q, sw13_s, sw2_q, sw2_s = (t[E] for t in stacked)
@@ -637,6 +639,9 @@ def main():
     ap.add_argument('--warmup', type=int, default=5)
     ap.add_argument('--workloads', default='gdn,gdn_single,gdn_fused,gdn_fused_norm,conv1d,moe_decode,router_decode,index_scores,index_scores_fp8,topk_select,mla,mla_paged,mla_fp8_cache,moe_prefill,router_prefill,rmsnorm_quant')
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--plain', action='store_true',
+                    help='MoE workloads: time the workload itself only, not its variants (shared expert, UE8M0 '
+                         'scales, requantisation forms), so that a profiler run sees one set of kernels')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run 3 plain device copies of 536 870 912 bytes (a kernel of known traffic, '
                          'for scaling the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)')
@@ -691,10 +696,10 @@ def main():
         elif name == 'mla_paged':
             results[name] = bench_mla(torch, capi, dev, args.steps, args.warmup, cpu, paged=True)
         elif name == 'moe_decode':
-            results[name] = bench_moe(torch, capi, dev, args.steps, args.warmup, cpu, prefill=False)
+            results[name] = bench_moe(torch, capi, dev, args.steps, args.warmup, cpu, prefill=False, plain=args.plain)
         elif name == 'moe_prefill':
             results[name] = bench_moe(torch, capi, dev, max(2, args.steps // 4), max(1, args.warmup // 2), cpu,
-                                      prefill=True)
+                                      prefill=True, plain=args.plain)
         else:
             sys.exit(f'bench.py: unknown workload {name}')
         torch.cuda.empty_cache()
