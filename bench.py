@@ -34,11 +34,24 @@ FP8_PEAK_TFLOPS = 5033.0
 METRIC = "GB/s & % HBM peak (GDN/MoE/MLA decode); fp8 TFLOP/s % MFMA peak (MoE prefill)"
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled
-# by the same counters read on a plain 512 MiB copy kernel (FETCH_SIZE x 1.99981, WRITE_SIZE x 1,
+# by the same counters read on a plain 512 MiB copy kernel (FETCH_SIZE x 1.99986, WRITE_SIZE x 1,
 # both in KiB); the counter summary is profiles/all_workloads_hbm_traffic_pmc.md.
 # None = not measured.
-MEASURED_TRAFFIC = {'gdn': 1085972770, 'moe_decode': 6664643628, 'mla': 223326108, 'index_scores': 553871480,
-                    'index_scores_fp8': 289779791, 'moe_prefill': 11230161000, 'mla_fp8_cache': 172870467}
+# Stamp: taken from the library as built from the sources of this tree (fp16 expert outputs in the prefill down
+# GEMM, bf16 matrix core in the decode gate/up GEMM); a change to a kernel's data movement needs a new run of
+# the two commands in that file.
+MEASURED_TRAFFIC = {'gdn': 1085846000, 'moe_decode': 6664690000, 'mla': 224332000, 'index_scores': 553927000,
+                    'index_scores_fp8': 289777000, 'moe_prefill': 11426305000, 'mla_fp8_cache': 172866000,
+                    'topk_select': 9216000}
+# Matrix-pipe occupancy of the dominant kernels from rocprofv3 --pmc (SQ_VALU_MFMA_BUSY_CYCLES over 1024 SIMDs x
+# GRBM_GUI_ACTIVE cycles per XCD, the timed launches of bench.py's own loop; the derived MfmaUtil counter reads
+# 39.6 / 33.5 / 22.3 %) and the clock by GRBM_GUI_ACTIVE / 8 / duration in the same run; the summary is
+# profiles/moe_prefill_mla_matrix_core_counters_pmc.md. Measured figures of that run, not of this one.
+MEASURED_MFMA = {
+    'moe_prefill': dict(mfma_busy=0.415, clock_ghz=1.92, kernel='moe_tiled_gemm_kernel<true> (gate/up)',
+                        mfma_busy_down=0.351, clock_ghz_down=1.75),
+    'mla': dict(mfma_busy=0.227, clock_ghz=2.07, kernel='sparse_mla_split8_kernel<false>'),
+}
 
 
 SETTLE_SECONDS = 0.05
@@ -416,7 +429,7 @@ def bench_topk_select(torch, capi, dev, steps, warmup, cpu_baseline):
                  "seed 20259 (one workgroup per request)",
         value=work / sec / 1e9, unit="GB/s", ms_per_step=sec * 1e3, dtype="u32", kernel="topk_select_kernel",
         roofline=dict(bound="hbm", achieved=work / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
-                      frac=work / sec / 1e9 / HBM_PEAK_GBS, traffic=None),
+                      frac=work / sec / 1e9 / HBM_PEAK_GBS, traffic=MEASURED_TRAFFIC['topk_select']),
         algorithmic_bytes=work)
     if cpu_baseline:
         cores = len(os.sched_getaffinity(0))
@@ -457,7 +470,8 @@ def bench_mla(torch, capi, dev, steps, warmup, cpu_baseline, paged=False):
                  ("; cache held as one pool of 64-row pages behind a block table" if paged else ""),
         value=work / sec / 1e9, unit="GB/s", ms_per_step=sec * 1e3, dtype="bf16", kernel="sparse_mla_split8_kernel",
         roofline=dict(bound="hbm", achieved=work / sec / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
-                      frac=work / sec / 1e9 / HBM_PEAK_GBS, traffic=None if paged else MEASURED_TRAFFIC['mla']),
+                      frac=work / sec / 1e9 / HBM_PEAK_GBS, traffic=None if paged else MEASURED_TRAFFIC['mla'],
+                      **({} if paged else MEASURED_MFMA['mla'])),
         algorithmic_bytes=work, tflops=flops / sec / 1e12)
     if cpu_baseline and not paged:
         cores = len(os.sched_getaffinity(0))
@@ -562,7 +576,8 @@ def bench_moe(torch, capi, dev, steps, warmup, cpu_baseline, prefill, plain=Fals
             value=flops / sec / 1e12, unit="TFLOP/s", ms_per_step=sec * 1e3, dtype="f8e4m3",
             kernel="moe_tiled_gemm_kernel",
             roofline=dict(bound="mfma", achieved=flops / sec / 1e12, peak=FP8_PEAK_TFLOPS, unit="TFLOP/s",
-                          frac=flops / sec / 1e12 / FP8_PEAK_TFLOPS, traffic=MEASURED_TRAFFIC['moe_prefill']),
+                          frac=flops / sec / 1e12 / FP8_PEAK_TFLOPS, traffic=MEASURED_TRAFFIC['moe_prefill'],
+                          **MEASURED_MFMA['moe_prefill']),
             algorithmic_flops=flops, active_experts=n_active)
     else:
         res = dict(
