@@ -65,9 +65,13 @@ typedef __attribute__((address_space(3))) void* lds_void_ptr;
 // position of 16-byte chunk `chunk` of row `row` inside a tile (in 16-byte units). A row is 1152
 // bytes = 4.5 x 256, so two consecutive rows share a row of the 64 LDS banks like rows of 128
 // bytes would; a ds_read_b128 serves 16 consecutive lanes per cycle, so among 16 consecutive
-// tile rows the 8 of equal parity must use 8 different chunk positions: the swizzle term is
-// (row >> 1) & 7 (with row & 7 the K operand reads ran at 2/3 of the conflict-free rate).
-__device__ __forceinline__ int row_swizzle(int row) { return (row >> 1) & 7; }
+// tile rows the 8 of equal parity must use 8 different chunk positions: the swizzle term is a
+// permutation of (row >> 1) & 7 (with row & 7 the K operand reads ran at 2/3 of the conflict-free rate).
+// The permutation is a rotation right by one bit, so that rows 2 apart differ in bit 2 of the term: a
+// transposing 8-byte read of the V^T operand takes 64 bytes from each of 4 consecutive rows per 32 lanes,
+// and rows of equal parity must take them from different halves of a 128-byte stretch (with the plain
+// (row >> 1) & 7 every such read cost two more LDS cycles, a fifth of the kernel's LDS time).
+__device__ __forceinline__ int row_swizzle(int row) { return ((row & 2) << 1) | ((row >> 2) & 3); }
 __device__ __forceinline__ int swizzled_slot(int row, int chunk) {
     return row * ROW_CHUNKS + ((chunk & ~7) | ((chunk ^ row_swizzle(row)) & 7));
 }
@@ -141,8 +145,8 @@ constexpr float FRAME_SLACK = 0.f;
 struct LaneOffsets {
     uint32_t qk[4];  // K operand of k-step ks: qk[ks & 3] + (ks >> 2) * 128
     uint32_t pv[2];  // V^T operand of dv tile t, k-step ks, half-read rr:
-                     //   (pv[t & 1] ^ 64*rr) + (16*ks + 8*rr) * ROW_BYTES + (t >> 1) * 128
-                     // (8 rows further down the swizzle term has bit 2 flipped)
+                     //   (pv[t & 1] ^ 32*rr) + (16*ks + 8*rr) * ROW_BYTES + (t >> 1) * 128
+                     // (8 rows further down the swizzle term has bit 1 flipped)
 };
 
 __device__ __forceinline__ LaneOffsets make_lane_offsets(int lane) {
@@ -281,7 +285,7 @@ __device__ __forceinline__ void process_tile(const uint4* tile, const int* s_idx
 #pragma unroll
         for (int rr = 0; rr < 2; ++rr) {
             dst[rr] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (lds_s4)(base + (off.pv[t & 1] ^ (64 * rr)) + (16 * ks + 8 * rr) * ROW_BYTES + (t >> 1) * 128));
+                (lds_s4)(base + (off.pv[t & 1] ^ (32 * rr)) + (16 * ks + 8 * rr) * ROW_BYTES + (t >> 1) * 128));
         }
     };
 #pragma unroll
@@ -519,7 +523,7 @@ __device__ __forceinline__ void gather_prepare(uint32_t (&off)[GATHER_INSTR], co
 #pragma unroll
     for (int i = 0; i < GATHER_INSTR; ++i) {
         const int key = *reinterpret_cast<const int*>(keys + (e[i] >> 16));
-        off[i] = (uint32_t)key * (uint32_t)ROW_BYTES + ((e[i] & 0xffffu) ^ ((quarter & 1) << 6));
+        off[i] = (uint32_t)key * (uint32_t)ROW_BYTES + ((e[i] & 0xffffu) ^ ((quarter & 1) << 5));
         if (has_padding && key < 0) off[i] = GATHER_MASKED;
     }
 }
@@ -665,9 +669,19 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
     const int dh = wave & 1;   // which slices of d (QK^T) and which half of dv (PV) this wavefront owns
     const int hg = wave >> 1;  // 32-head group
     const int group = wave >> 2;
-    const int split = blockIdx.x;
     const int n_splits = gridDim.x;
-    const int b = blockIdx.y;
+    int split = blockIdx.x;
+    int b = blockIdx.y;
+    // Consecutive workgroup ids go round-robin to the 8 XCDs, each with its own L2. With the plain mapping the
+    // splits of a request land on four XCDs and each of them fetches the request's 147 KB of Q; with a batch
+    // that is a multiple of 8 the splits of request b all run on XCD b % 8 (one fetch of Q per XCD, and the
+    // request's partials are written through one L2, where the merge kernel looks for them).
+    if ((gridDim.y & 7) == 0) {
+        const int linear = blockIdx.x + gridDim.x * blockIdx.y;
+        const int j = linear >> 3;
+        split = j % n_splits;
+        b = (linear & 7) + 8 * (j / n_splits);
+    }
     const int head0 = blockIdx.z * 128 + hg * 32;
     const int half = lane >> 5;
 
@@ -708,7 +722,7 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
     if (tid == 0) s_first_masked_tile = n_tiles;
     for (int c = tid; c < (FP8 ? 0 : GATHER_TAB); c += 512) {  // (the e4m3 gather computes its offsets itself)
         const int row = c / ROW_CHUNKS;  // 0..7; the tile row is 8*quarter + row: for odd quarters the
-        const int pos = c - row * ROW_CHUNKS;  // swizzle term has bit 2 flipped (gather_prepare)
+        const int pos = c - row * ROW_CHUNKS;  // swizzle term has bit 1 flipped (gather_prepare)
         const int chunk = (pos & ~7) | ((pos ^ row_swizzle(row)) & 7);
         s_gather_tab[c] = ((uint32_t)(4 * row) << 16) | (uint32_t)(chunk * 16);
     }
@@ -780,7 +794,7 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
     SoftmaxState st{-INFINITY, 0.f};
     const LaneOffsets off = make_lane_offsets(lane);
     // K operand of local step l: qk_l[l & 1] + (l >> 1) * 128
-    // V^T operand of local dv tile tl: (pv_l[tl & 1] ^ 64*rr) + (16*ks + 8*rr) * ROW_BYTES + (tl >> 1) * 128
+    // V^T operand of local dv tile tl: (pv_l[tl & 1] ^ 32*rr) + (16*ks + 8*rr) * ROW_BYTES + (tl >> 1) * 128
     const uint32_t qk_l[2] = {dh ? off.qk[2] : off.qk[0], dh ? off.qk[3] : off.qk[1]};
     const uint32_t pv_l[2] = {off.pv[0] + 512u * dh, off.pv[1] + 512u * dh};
     floatx4* my_xchg = &s_xchg[wave][0];
@@ -955,7 +969,7 @@ __global__ __launch_bounds__(512) void sparse_mla_split8_kernel(
 #pragma unroll
                 for (int rr = 0; rr < 2; ++rr) {
                     dst[j][rr] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (lds_s4)(base + (pv_l[tl & 1] ^ (64 * rr)) + (16 * ks + 8 * rr) * ROW_BYTES + (tl >> 1) * 128));
+                        (lds_s4)(base + (pv_l[tl & 1] ^ (32 * rr)) + (16 * ks + 8 * rr) * ROW_BYTES + (tl >> 1) * 128));
                 }
             }
         };
@@ -1046,8 +1060,18 @@ __global__ __launch_bounds__(256) void sparse_mla_merge_kernel(const PART* __res
     typedef PART partx8 __attribute__((ext_vector_type(8)));
     typedef float floatx8 __attribute__((ext_vector_type(8)));
     const int lane = threadIdx.x & 63;
-    const int h = blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int b = blockIdx.y;
+    int hg = blockIdx.x;
+    int b = blockIdx.y;
+#ifndef MLA_MERGE_PLAIN_MAP
+    // request b on XCD b % 8, where the split kernel wrote its partials (see there)
+    if ((gridDim.y & 7) == 0) {
+        const int linear = blockIdx.x + gridDim.x * blockIdx.y;
+        const int j = linear >> 3;
+        hg = j % (int)gridDim.x;
+        b = (linear & 7) + 8 * (j / (int)gridDim.x);
+    }
+#endif
+    const int h = hg * 4 + (threadIdx.x >> 6);
     const size_t base = (size_t)b * n_splits * n_heads + h;
     floatx8 o = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     float wsum = 0.f;
