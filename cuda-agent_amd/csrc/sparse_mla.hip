@@ -1081,8 +1081,12 @@ __global__ __launch_bounds__(256) void sparse_mla_merge_kernel(const PART* __res
         for (int j = 0; j < BATCH; ++j) {
             // (splits past the end repeat the last one; their weight is 0)
             const int s = s0 + j < n_splits ? s0 + j : n_splits - 1;
+#ifdef MLA_MERGE_PLAIN_LOADS
+            rows[j] = *(reinterpret_cast<const partx8*>(o_part + (base + (size_t)s * n_heads) * D_V) + lane);
+#else
             rows[j] = __builtin_nontemporal_load(
                 reinterpret_cast<const partx8*>(o_part + (base + (size_t)s * n_heads) * D_V) + lane);
+#endif
         }
     };
     // the first rows are requested before anything depends on the log-sum-exps
