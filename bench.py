@@ -40,17 +40,17 @@ METRIC = "GB/s & % HBM peak (GDN/MoE/MLA decode); fp8 TFLOP/s % MFMA peak (MoE p
 # Stamp: taken from the library as built from the sources of this tree (fp16 expert outputs in the prefill down
 # GEMM, bf16 matrix core in the decode gate/up GEMM); a change to a kernel's data movement needs a new run of
 # the two commands in that file.
-MEASURED_TRAFFIC = {'gdn': 1085846000, 'moe_decode': 6664690000, 'mla': 224332000, 'index_scores': 553927000,
-                    'index_scores_fp8': 289777000, 'moe_prefill': 11426305000, 'mla_fp8_cache': 172866000,
+MEASURED_TRAFFIC = {'gdn': 1085846000, 'moe_decode': 6664690000, 'mla': 196017000, 'index_scores': 553927000,
+                    'index_scores_fp8': 289777000, 'moe_prefill': 11426305000, 'mla_fp8_cache': 145212000,
                     'topk_select': 9216000}
 # Matrix-pipe occupancy of the dominant kernels from rocprofv3 --pmc (SQ_VALU_MFMA_BUSY_CYCLES over 1024 SIMDs x
 # GRBM_GUI_ACTIVE cycles per XCD, the timed launches of bench.py's own loop; the derived MfmaUtil counter reads
-# 39.6 / 33.5 / 22.3 %) and the clock by GRBM_GUI_ACTIVE / 8 / duration in the same run; the summary is
+# 39.6 / 33.5 / 22.9 %) and the clock by GRBM_GUI_ACTIVE / 8 / duration in the same run; the summary is
 # profiles/moe_prefill_mla_matrix_core_counters_pmc.md. Measured figures of that run, not of this one.
 MEASURED_MFMA = {
     'moe_prefill': dict(mfma_busy=0.415, clock_ghz=1.92, kernel='moe_tiled_gemm_kernel<true> (gate/up)',
                         mfma_busy_down=0.351, clock_ghz_down=1.75),
-    'mla': dict(mfma_busy=0.227, clock_ghz=2.07, kernel='sparse_mla_split8_kernel<false>'),
+    'mla': dict(mfma_busy=0.238, clock_ghz=2.03, kernel='sparse_mla_split8_kernel<false>'),
 }
 
 
