@@ -50,7 +50,9 @@ def check(capi, q, kv, idx, config, ref):
 
 @pytest.mark.parametrize('config', [0, 1, 2, 5])
 @pytest.mark.parametrize('shape', [(2, 128, 300, 96), (3, 32, 100, 33), (1, 64, 512, 257),
-                                   (2, 128, 4096, 2048), (1, 256, 200, 64), (5, 128, 64, 1)])
+                                   (2, 128, 4096, 2048), (1, 256, 200, 64), (5, 128, 64, 1),
+                                   # batches that are multiples of 8: the splits of a request share an XCD
+                                   (8, 128, 600, 200), (16, 256, 300, 130), (8, 128, 2048, 1024), (24, 128, 90, 70)])
 def test_matches_oracle(capi, dev, shape, config):
     B, H, N, topk = shape
     gen = torch.Generator().manual_seed(B * 1000 + topk)
