@@ -489,6 +489,42 @@ def test_rejects_bad_arguments(capi, dev):
         capi.moe_fp8_launch(out, *dts, big, top_k=8)      # top_k > n_experts
 
 
+BINDING_AT_FULL_SIZE = r"""
+import sys, torch
+sys.path.insert(0, {repo!r}); sys.path.insert(0, {tests!r}); sys.path.insert(0, {ws!r})
+import __graft_entry__ as entry
+entry.load_package()
+from cuda_agent_amd import capi
+import cuda_extension                      # the workspace's module, built by utils/compile.py
+from test_moe_gpu import full_size_layer
+dev = torch.device('cuda:0')
+dts = full_size_layer(dev, 8192, 20254, n_biased=16)
+for tokens in (64, 8192):                   # configs[2] and configs[4] on one set of weights
+    x, logits = dts[0][:tokens].contiguous(), dts[1][:tokens].contiguous()
+    got = cuda_extension.moe_fp8_forward(x, logits, *dts[2:], 8)
+    want = torch.empty(tokens, 7168, dtype=torch.bfloat16, device=dev)
+    ws = torch.empty(capi.moe_workspace_bytes(tokens, 7168, 2048, 256, 8), dtype=torch.uint8, device=dev)
+    capi.moe_fp8_launch(want, x, logits, *dts[2:], ws, top_k=8)
+    torch.cuda.synchronize()
+    assert torch.isfinite(got.float()).all() and got.float().abs().mean().item() > 0
+    assert torch.equal(got, want), tokens
+    print('binding == C ABI at', tokens, 'tokens')
+"""
+
+
+def test_workspace_binding_at_the_workload_sizes():
+    """`moe_fp8_forward` of the workspace extension (the pybind binding `ModelNew` calls) on configs[2] and
+    configs[4] sized inputs: bit-equal to the C-ABI launcher, whose output the two full-size tests above hold
+    against the oracle. In a process of its own: every workspace's module is called `cuda_extension`."""
+    root = Path(__file__).resolve().parent.parent
+    ws = root / 'cuda-agent_amd' / 'workspaces' / 'moe_fp8'
+    assert (ws / 'cuda_extension.so').exists(), 'workspace extension not built'
+    script = BINDING_AT_FULL_SIZE.format(repo=str(root), tests=str(root / 'tests'), ws=str(ws))
+    out = subprocess.run([sys.executable, '-c', script], capture_output=True, text=True, timeout=900)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert 'binding == C ABI at 64 tokens' in out.stdout and 'binding == C ABI at 8192 tokens' in out.stdout
+
+
 def test_workspace_verification_flow():
     """`python3 -m utils.verification` from inside the workspace, as its user runs it (reduced
     layer: the full one spends minutes drawing 11 GB of weights on the host)."""
