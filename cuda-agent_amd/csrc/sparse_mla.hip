@@ -533,7 +533,8 @@ __device__ __forceinline__ void gather_issue(uint4* tile, const char* kv_b, uint
     uint4* dst = tile + quarter * GATHER_TAB + i * 64;
     if (!has_padding || off != GATHER_MASKED) {
         const uint32_t lds_base = (uint32_t)(size_t)((lds_void_ptr)dst);
-        asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+        // (non-temporal: a selected row is read once per launch; 66.6 -> 65.1 us per step)
+        asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1 nt"
                      :
                      : "v"(off), "s"(kv_b), "s"(lds_base)
                      : "memory", "m0");
@@ -575,7 +576,7 @@ __device__ __forceinline__ void gather_quarter_fp8(uint4* tile, const char* kv_b
 #pragma unroll
     for (int k = 0; k < FP8_GATHER_INSTR; ++k) {
         if (64 * k + 64 <= FP8_STAGE_CHUNKS || lane < FP8_STAGE_CHUNKS - 64 * k) {
-            asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+            asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1 nt"
                          :
                          : "v"(off[k]), "s"(kv_b), "s"(lds_base + 1024u * k)
                          : "memory", "m0");
