@@ -44,3 +44,23 @@ def test_no_committed_file_reads_the_scratch_folder():
         if re.search(r'''["'/]_work["'/]''', path.read_text(errors='replace')):
             offenders.append(str(path.relative_to(REPO)))
     assert not offenders, offenders
+
+
+def test_measured_constants_of_bench_are_the_figures_of_the_committed_profiles():
+    """bench.py carries HBM traffic and matrix-pipe occupancy as constants taken from rocprofv3 counter runs;
+    each must be a figure of the committed summary it names, so that one cannot change without the other."""
+    import ast
+    src = (REPO / 'bench.py').read_text()
+    tree = ast.parse(src)
+    values = {}
+    for node in tree.body:
+        if isinstance(node, ast.Assign) and getattr(node.targets[0], 'id', '') in ('MEASURED_TRAFFIC', 'MEASURED_MFMA'):
+            values[node.targets[0].id] = ast.literal_eval(ast.unparse(node.value).replace('dict(', 'dict(')) \
+                if node.targets[0].id == 'MEASURED_TRAFFIC' else ast.unparse(node.value)
+    traffic_md = (REPO / 'profiles' / 'all_workloads_hbm_traffic_pmc.md').read_text()
+    for name, nbytes in values['MEASURED_TRAFFIC'].items():
+        spaced = f'{nbytes:,}'.replace(',', ' ')
+        assert spaced in traffic_md, (name, spaced)
+    counters_md = (REPO / 'profiles' / 'moe_prefill_mla_matrix_core_counters_pmc.md').read_text()
+    for figure in re.findall(r'mfma_busy(?:_down)?=([0-9.]+)', values['MEASURED_MFMA']):
+        assert figure in counters_md, figure
