@@ -622,16 +622,18 @@ def bench_moe(torch, capi, dev, steps, warmup, cpu_baseline, prefill, plain=Fals
     res['with_ue8m0_scales'] = dict(
         ms_per_step=sec3 * 1e3, unit=res['unit'], value=flops / sec3 / 1e12 if prefill else wbytes / sec3 / 1e9,
         note="moe_fp8_launcher with config 32: the same workload with every block scale a power of two")
-    # how the intermediate is requantised: the decode step runs its gate/up GEMM on the bf16 matrix core (codes
-    # agree with an fp32 evaluation), config 512 puts it on the e4m3 one; the prefill step runs the e4m3 matrix
-    # core, config 256 adds the pass that recomputes the elements near a rounding boundary
-    other = 256 if prefill else 512
-    sec4 = timed_launches(
-        torch, lambda i: capi.moe_fp8_launch(out, x, logits, w13_q, w13_s, w2_q, w2_s, ws3, config=other),
-        max(2, steps // 2), 1)
-    res['with_exact_requantisation_pass' if prefill else 'gate_up_on_e4m3_matrix_core'] = dict(
-        ms_per_step=sec4 * 1e3, unit=res['unit'], value=flops / sec4 / 1e12 if prefill else wbytes / sec4 / 1e9,
-        note=f"moe_fp8_launcher with config {other}")
+    # how the intermediate is requantised. Decode: the gate/up GEMM runs on the bf16 matrix core (codes agree with
+    # an fp32 evaluation), config 512 puts it on the e4m3 one. Prefill: e4m3 matrix core with the codes of the large
+    # elements repaired in the epilogue; config 256 runs gate/up on the bf16 matrix core instead (every code
+    # exact), config 512 leaves the e4m3 matrix core's codes as they come.
+    for key, other in ((('gate_up_on_bf16_matrix_core', 256), ('e4m3_matrix_core_without_repair', 512)) if prefill
+                       else (('gate_up_on_e4m3_matrix_core', 512),)):
+        sec4 = timed_launches(
+            torch, lambda i: capi.moe_fp8_launch(out, x, logits, w13_q, w13_s, w2_q, w2_s, ws3, config=other),
+            max(2, steps // 2), 1)
+        res[key] = dict(
+            ms_per_step=sec4 * 1e3, unit=res['unit'], value=flops / sec4 / 1e12 if prefill else wbytes / sec4 / 1e9,
+            note=f"moe_fp8_launcher with config {other}")
     del ws3
     if cpu_baseline:
         n_tok = 4
@@ -713,10 +715,11 @@ def main():
         elif name == 'moe_decode':
             results[name] = bench_moe(torch, capi, dev, args.steps, args.warmup, cpu, prefill=False, plain=args.plain)
         elif name == 'moe_prefill':
-            results[name] = bench_moe(torch, capi, dev, max(2, args.steps // 4), max(1, args.warmup // 2), cpu,
+            results[name] = bench_moe(torch, capi, dev, args.steps, max(1, args.warmup // 2), cpu,
                                       prefill=True, plain=args.plain)
         else:
             sys.exit(f'bench.py: unknown workload {name}')
+        results[name].setdefault('steps_timed', args.steps)
         torch.cuda.empty_cache()
 
     head_name = 'gdn' if 'gdn' in results else wanted[0]
@@ -729,6 +732,12 @@ def main():
                    "settle": f"{SETTLE_SECONDS} s of untimed launches before the warm-up steps of every workload"},
         "roofline": head['roofline'],
     }
+    # the four workloads the targets are stated on, inside the headline's roofline object
+    line["roofline"] = dict(head['roofline'], per_workload={
+        k: dict(ms_per_step=results[k]['ms_per_step'], frac=results[k]['roofline']['frac'],
+                achieved=results[k]['roofline']['achieved'], unit=results[k]['roofline']['unit'],
+                steps_timed=results[k]['steps_timed'])
+        for k in ('gdn', 'moe_decode', 'mla', 'moe_prefill') if k in results})
     if 'cpu_baseline' in head:
         line["cpu_baseline"] = head['cpu_baseline']
     shown = ('workload', 'value', 'unit', 'ms_per_step', 'dtype', 'roofline', 'cpu_baseline')

@@ -73,7 +73,7 @@ SIGNATURES = {
     'moe_fp8_fused_shared_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int,
                                              c_int, c_int, c_int, c_int, _P]),
     'moe_fp8_workspace_bytes': (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
-    'moe_fp8_workspace_layout': (None, [_P, c_int, c_int, c_int, c_int, c_int]),
+    'moe_fp8_workspace_layout': (c_int, [_P, c_int, c_int, c_int, c_int, c_int, c_int]),
     'moe_fp8_uses_tiled_gemms': (c_int, [c_int, c_int, c_int, c_int, c_int, c_int]),
     'moe_fp8_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int,
                                 c_int, c_int, c_int, _P]),
@@ -522,7 +522,7 @@ def topk_select_launch(idx_out, scores, lengths=None, stream=None):
 
 
 MOE_WORKSPACE_FIELDS = ('ids', 'weights', 'expert_offsets', 'sorted_pairs', 'pair_pos', 'x_q', 'x_s',
-                        'h_q', 'h_s', 'y', 'h_marks', 'y_scale')
+                        'h_q', 'h_s', 'y', 'y_scale')
 
 
 def moe_workspace_bytes(tokens, hidden, inter, n_experts, top_k=8):
@@ -530,10 +530,14 @@ def moe_workspace_bytes(tokens, hidden, inter, n_experts, top_k=8):
 
 
 def moe_workspace_views(workspace, tokens, hidden, inter, n_experts, top_k=8):
-    """Typed views of the intermediate buffers inside a workspace tensor (uint8, 1-D)."""
+    """Typed views of the intermediate buffers inside a workspace tensor (uint8, 1-D). ``y`` is laid out as
+    fp32 rows; when the layer ran the LDS-tiled GEMMs (``moe_fp8_uses_tiled_gemms`` returns 1) it holds fp16 rows
+    with the scales in ``y_scale`` instead and must be read through ``moe_expert_outputs``."""
     import torch
     offs = (c_size_t * len(MOE_WORKSPACE_FIELDS))()
-    library().moe_fp8_workspace_layout(offs, tokens, hidden, inter, n_experts, top_k)
+    n = library().moe_fp8_workspace_layout(offs, len(MOE_WORKSPACE_FIELDS), tokens, hidden, inter, n_experts, top_k)
+    _require(n == len(MOE_WORKSPACE_FIELDS), f'moe_fp8_workspace_layout has {n} fields, this module knows '
+                                             f'{len(MOE_WORKSPACE_FIELDS)}')
     pairs = tokens * top_k
     spec = {
         'ids': (torch.int32, (tokens, top_k)), 'weights': (torch.float32, (tokens, top_k)),
@@ -541,7 +545,7 @@ def moe_workspace_views(workspace, tokens, hidden, inter, n_experts, top_k=8):
         'pair_pos': (torch.int32, (pairs,)), 'x_q': (torch.float8_e4m3fn, (tokens, hidden)),
         'x_s': (torch.float32, (tokens, hidden // 128)), 'h_q': (torch.float8_e4m3fn, (pairs, inter)),
         'h_s': (torch.float32, (pairs, inter // 128)), 'y': (torch.float32, (pairs, hidden)),
-        'h_marks': (torch.uint8, (pairs, inter)), 'y_scale': (torch.float32, (pairs, (hidden + 255) // 256)),
+        'y_scale': (torch.float32, (pairs, (hidden + 255) // 256)),
     }
     views = {}
     for name, off in zip(MOE_WORKSPACE_FIELDS, offs):

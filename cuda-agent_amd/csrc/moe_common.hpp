@@ -27,37 +27,63 @@ constexpr int CONFIG_SHARED_SLOT = 64;
 // more pairs than the others (the shared expert above): dispatch its workgroups first.
 constexpr int CONFIG_LAST_EXPERT_FIRST = 128;
 
-// config bits of the layer and of the gate/up stage that decide how exactly h = silu(g) * u is requantised.
+// config bits of the layer and of the gate/up stage that decide how h = silu(g) * u is requantised.
 // The e4m3 matrix core adds the products of a 128-block with about 16 significant bits, so its g and u carry
 // an error in the 5th digit and about one code of h in a thousand lands on the other side of a rounding
-// boundary (one code step, 6-12 % of that element; the group's scale moves in the 5th digit as well).
+// boundary (one code step, 6-12 % of that element; the group's scale moves in the 5th digit as well). One such
+// step on an element near its group's maximum moves single outputs of the layer by up to 3 % of their rms.
 //  * The streaming gate/up GEMM (few pairs per expert, bound by the weight stream) converts the codes to bf16
 //    in registers and uses the bf16 matrix core, whose sums are exact to fp32 accuracy: its h agrees with an
 //    fp32 evaluation. CONFIG_APPROX_REQUANT puts it on the e4m3 matrix core.
-//  * The tiled gate/up GEMM (many pairs per expert, bound by the matrix core) stays on the e4m3 instruction.
-//    With CONFIG_EXACT_REQUANT its epilogue marks every element whose scaled value lies within the error band
-//    of a rounding boundary and every element that may be the group's maximum, and a second kernel
-//    (moe_requant_fix_launcher) recomputes those pre-activations as plain dot products, takes the scale from
-//    the exact maximum and rewrites the marked codes. That pass re-reads two weight rows per marked element:
-//    negligible at a few hundred pairs, more than the whole layer at thousands of pairs per expert, so it is
-//    off unless asked for. Bits 10-11 scale the width of its band: 0 the default, 1 half, 2 twice, 3 four
-//    times as wide.
+//  * The tiled gate/up GEMM (many pairs per expert, bound by the matrix core):
+//      default: e4m3 matrix core, and the epilogue repairs the codes that matter. It marks every element whose
+//        scaled magnitude reaches 2^s code units (s = bits 12-15; 0: default_requant_significance, which is 7 at
+//        the sizes this form is meant for: 128 of 448, i.e. the two highest binades, where one code step is 16 or
+//        32 units) and lies within the error band of a rounding boundary,
+//        and recomputes those pre-activations, and the candidates for the maximum of their group of 128, as
+//        plain dot products; the group's scale then comes from the exact maximum and the marked codes from
+//        the exact values. Smaller elements keep the matrix core's code (a step of at most 8 units there).
+//      CONFIG_EXACT_REQUANT: bf16 matrix core (twice the matrix-core time): every code as an fp32
+//        evaluation gives it, as in the streaming form.
+//      CONFIG_APPROX_REQUANT: e4m3 matrix core, codes as they come.
+//    Bits 10-11 scale the width of the band: 0 the default, 1 half, 2 twice, 3 four times as wide.
 constexpr int CONFIG_EXACT_REQUANT = 256;
 constexpr int CONFIG_APPROX_REQUANT = 512;
 constexpr int CONFIG_BAND_SHIFT = 10;
 constexpr int CONFIG_BAND_MASK = 3 << CONFIG_BAND_SHIFT;
-constexpr int CONFIG_REQUANT_BITS = CONFIG_EXACT_REQUANT | CONFIG_APPROX_REQUANT | CONFIG_BAND_MASK;
+constexpr int CONFIG_SIGNIF_SHIFT = 12;
+constexpr int CONFIG_SIGNIF_MASK = 15 << CONFIG_SIGNIF_SHIFT;
+constexpr int CONFIG_REQUANT_BITS = CONFIG_EXACT_REQUANT | CONFIG_APPROX_REQUANT | CONFIG_BAND_MASK | CONFIG_SIGNIF_MASK;
 
-// marks of one element of h (one byte per element, same layout as h_q)
+// marks of one element of h
 constexpr uint32_t MARK_NEAR = 1;       // the scaled value may round to either of two codes
 constexpr uint32_t MARK_CANDIDATE = 2;  // the element may be the largest magnitude of its group
+
+// Significance level s the layer uses when the config names none: elements of at least 2^s code units are
+// repaired. One code step of an element moves an output by an amount that shrinks, relative to the output's rms,
+// with the square root of the number of terms an output sums (inter * top_k): 2^7 at inter * top_k = 16384
+// (a step of at most 8 units below it, which measured moves no output by more than 2e-3 of the rms there),
+// half of that for every factor of four fewer terms, never below 2^3.
+inline int default_requant_significance(int inter, int top_k) {
+    int s = 7;
+    for (long terms = (long)inter * top_k; terms < 16384 && s > 3; terms *= 4) --s;
+    return s;
+}
+
+// smallest scaled magnitude, in e4m3 code units, an element must reach for MARK_NEAR (config with the
+// significance bits set)
+inline float requant_min_magnitude(int config) {
+    const int sig = (config & CONFIG_SIGNIF_MASK) >> CONFIG_SIGNIF_SHIFT;
+    return (float)(1 << (sig ? sig : 7));
+}
 
 // Error of a gate/up pre-activation as the e4m3 matrix core computes it, as a multiple of the root mean square
 // of the pair's 256 pre-activations of the row block. Measured on gfx950: the partial of one 128-block is off by
 // 1.4e-6 of the block's sum of |products| on average (13 times that at most), without a preferred sign. For
 // operands without a common sign the errors of the K/128 blocks add up like a random walk while the result
 // grows with sqrt(K) as well, so one standard deviation of the error is about 1.3e-5 of the root mean square
-// of the results whatever K is; the band takes 4.5 of them (times `width`).
+// of the results whatever K is; the band takes 4.5 of them (times `width`). This is an error model, not a
+// bound: operands of one sign throughout, for which the error grows with K, are outside it.
 inline float requant_error_coefficient(int config) {
     static const float width[4] = {1.f, 0.5f, 2.f, 4.f};
     return width[(config & CONFIG_BAND_MASK) >> CONFIG_BAND_SHIFT] * 4.5f * 1.3e-5f;
@@ -68,7 +94,7 @@ inline float requant_error_coefficient(int config) {
 // scale / amax the group's scale and maximum as computed, err the error bound of g and of u, dh_max a bound of
 // the error of any element of the group, scale_uncertain whether the exact maximum may give another scale.
 __device__ __forceinline__ uint32_t requant_marks(float h, float sg, float u, float scale, float amax, float err,
-                                                  float dh_max, bool scale_uncertain) {
+                                                  float dh_max, bool scale_uncertain, float v_min = 0.f) {
     // |d silu / d g| <= 1.1
     const float dh = (1.1f * fabsf(u) + fabsf(sg)) * err;
     const float v = fminf(fabsf(h) / scale, E4M3_MAX);
@@ -77,7 +103,7 @@ __device__ __forceinline__ uint32_t requant_marks(float h, float sg, float u, fl
     const float lo = fmaxf(v - tau, 0.f);
     const float hi = fminf(v + tau, E4M3_MAX);
     const int codes = __builtin_amdgcn_cvt_pk_fp8_f32(lo, hi, 0, false);
-    uint32_t m = ((codes ^ (codes >> 8)) & 0xff) != 0 ? MARK_NEAR : 0u;
+    uint32_t m = ((codes ^ (codes >> 8)) & 0xff) != 0 && hi >= v_min ? MARK_NEAR : 0u;
     if (scale_uncertain && fabsf(h) + 2.f * dh_max >= amax) m |= MARK_CANDIDATE;
     return m;
 }
@@ -116,7 +142,6 @@ struct Workspace {
     float* xs_t;          // [H/128][scale_stride] activation scales by sorted position, transposed
     float* hs_t;          // [I/128][scale_stride] the same for h
     int scale_stride;     // pairs rounded up to 256, plus 256 of padding
-    uint8_t* h_marks;     // [T*k*I] marks of the exact requantisation (MARK_*), rows in sorted order
     size_t bytes;
 };
 
@@ -149,7 +174,6 @@ inline Workspace carve_workspace(void* base, int tokens, int hidden, int inter, 
     w.tile_start = reinterpret_cast<int*>(take(((size_t)n_experts + 1) * 4));
     w.xs_t = reinterpret_cast<float*>(take((size_t)(hidden / GROUP) * w.scale_stride * 4));
     w.hs_t = reinterpret_cast<float*>(take((size_t)(inter / GROUP) * w.scale_stride * 4));
-    w.h_marks = reinterpret_cast<uint8_t*>(take(pairs * inter));
     w.y_scale = reinterpret_cast<float*>(take(pairs * ((hidden + 255) / 256) * 4));
     w.bytes = off;
     return w;

@@ -32,8 +32,11 @@ using namespace moe;
 
 typedef int intx8 __attribute__((ext_vector_type(8)));
 typedef int intx4 __attribute__((ext_vector_type(4)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
 typedef const __attribute__((address_space(3))) uint8_t* lds_bytes;
 typedef const __attribute__((address_space(3))) intx4* lds_x4;
@@ -66,6 +69,38 @@ __device__ __forceinline__ intx8 join(intx4 lo, intx4 hi) {
 // division were a tenth of a full tile's time in the gate/up epilogue)
 __device__ __forceinline__ float silu(float x) {
     return x * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
+}
+
+// 8 e4m3 codes (two dwords) -> 8 bf16, exactly (every e4m3 value is a bf16 value)
+__device__ __forceinline__ bf16x8 e4m3x8_to_bf16(int lo, int hi) {
+    const bf16x2 a = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, false);
+    const bf16x2 b = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, true);
+    const bf16x2 c = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, false);
+    const bf16x2 d = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, true);
+    return bf16x8{a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
+}
+
+// sum over 16 e4m3 pairs of a * b, in fp32 (the products are exact, the sum is rounded 15 times)
+__device__ __forceinline__ float dot16(intx4 a, intx4 b) {
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const floatx2 a0 = __builtin_amdgcn_cvt_pk_f32_fp8(a[j], false);
+        const floatx2 a1 = __builtin_amdgcn_cvt_pk_f32_fp8(a[j], true);
+        const floatx2 b0 = __builtin_amdgcn_cvt_pk_f32_fp8(b[j], false);
+        const floatx2 b1 = __builtin_amdgcn_cvt_pk_f32_fp8(b[j], true);
+        s = fmaf(a0[0], b0[0], s);
+        s = fmaf(a0[1], b0[1], s);
+        s = fmaf(a1[0], b1[0], s);
+        s = fmaf(a1[1], b1[1], s);
+    }
+    return s;
+}
+
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) v += __shfl_xor(v, d);
+    return v;
 }
 
 __device__ __forceinline__ void wait_all_loads() {
@@ -160,14 +195,14 @@ __device__ unsigned long long g_wg_trace[16384][3];
 // 2^(byte - 127)), the products of all K blocks add up in the accumulator itself, and the per-block
 // multiply-add on the VALU (128 per wavefront and K block) disappears.
 // FIX (gate/up only): the epilogue also writes the marks of the exact requantisation (moe_common.hpp).
-template <bool GATE_UP, bool UE8M0, bool FIX = false>
+template <bool GATE_UP, bool UE8M0, bool FIX = false, bool BF16 = false>
 __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
     const uint8_t* __restrict__ w_q, const float* __restrict__ w_s, const uint8_t* __restrict__ a_q,
     const float* __restrict__ as_t, const int* __restrict__ sorted_pairs,
     const int* __restrict__ expert_offsets, const int* __restrict__ tile_start,
     uint8_t* __restrict__ h_q, float* __restrict__ h_s, float* __restrict__ hs_t, float* __restrict__ y,
     float* __restrict__ y_scale, int K, int n_rows, int inter, int top_k, int n_experts, int scale_stride,
-    uint8_t* __restrict__ h_marks, float err_coef) {
+    float err_coef, float v_min) {
     __shared__ __attribute__((aligned(16))) uint8_t s_stage[2 * STAGE_BYTES];
 
     // Workgroup -> (row tile, pair tile). Consecutive workgroup ids go round-robin to the 8 XCDs,
@@ -300,6 +335,7 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
     //    VALU work hides behind the matrix pipeline with two partial accumulators only.
     // kb1, kb2: kb+1 and kb+2, or 0 past the end (harmless loads that keep the body branch-free;
     // the epilogue waits for them before it reuses the stages).
+    PHASE_TIMING_BEGIN();
     auto block = [&](auto nb_tag, auto half_tag, int kb, int kb1, int kb2) {
         constexpr int NB = decltype(nb_tag)::value;
         constexpr bool HALF = decltype(half_tag)::value != 0;  // a half tile (compile time: full tiles keep their code)
@@ -325,7 +361,7 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
                 A[1][s] = join(*(lds_x4)(st + a_row1 * GROUP + (rd ^ (64 * s))),
                                *(lds_x4)(st + a_row1 * GROUP + (rd ^ (64 * s) ^ 16)));
             }
-            read_b(0);
+            if constexpr (!BF16) read_b(0);
             bs = read_bs(0);
         }
         // every wavefront holds its A operands: the weight half of this stage may be refilled
@@ -361,6 +397,74 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
         }
         const float w0 = ws0[kb];
         const float w1 = ws1[kb];
+        if constexpr (BF16) {
+            // Gate/up on the bf16 matrix core: every e4m3 code is a bf16 value, and v_mfma_f32_32x32x16_bf16 adds
+            // the products of a 128-block to fp32 accuracy (the e4m3 instruction keeps about 16 bits), so that the
+            // requantised h agrees with an fp32 evaluation. A lane's 32 operand bytes of a k-step, eight at a time,
+            // are the operands of four such MFMAs (A and B take the same bytes of their lanes, so the products
+            // pair up the same k whichever order the matrix core walks them in).
+            // Schedule: the A operands are converted once per block (64 registers); per B tile the 8 MFMAs of A
+            // tile 0 run as one chain into p0, then the 8 of A tile 1 into p1. B arrives 16 bytes (two MFMAs) at
+            // a time, just in time, and is read and converted once per chain, so that only 8 + 8 registers hold B.
+            // The partial of one chain is promoted under the MFMAs of the next: per MFMA (32 cycles) the wavefront
+            // issues 4 conversions and 2 multiply-adds, which is what fits beside it.
+            bf16x8 Ab[2][8];
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+#pragma unroll
+                for (int s = 0; s < 2; ++s)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) Ab[a][4 * s + j] = e4m3x8_to_bf16(A[a][s][2 * j], A[a][s][2 * j + 1]);
+            // piece u (0..3) of B tile b: the 16 bytes that feed MFMAs 2u and 2u+1 of a chain
+            auto b_piece = [&](int b, int u) {
+                const lds_bytes bt = st + STAGE_A + (rh * 128 + b * 32) * GROUP;
+                return *(lds_x4)(bt + (rd ^ (64 * (u >> 1)) ^ (16 * (u & 1))));
+            };
+            floatx16 p0, p1;
+            float s0 = 0.f, s1_prev = 0.f;
+            intx4 q = b_piece(0, 0);
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {  // chain of A tile 0; p1 of the tile before is promoted meanwhile
+                    const bf16x8 f0 = e4m3x8_to_bf16(q[0], q[1]);
+                    const bf16x8 f1 = e4m3x8_to_bf16(q[2], q[3]);
+                    q = b_piece(b, (u + 1) & 3);
+                    p0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Ab[0][2 * u], f0, u == 0 ? floatx16{0} : p0, 0, 0, 0);
+                    if (b > 0) {
+#pragma unroll
+                        for (int i = 4 * u; i < 4 * u + 2; ++i) acc[1][b - 1][i] += p1[i] * s1_prev;
+                    }
+                    p0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Ab[0][2 * u + 1], f1, p0, 0, 0, 0);
+                    if (b > 0) {
+#pragma unroll
+                        for (int i = 4 * u + 2; i < 4 * u + 4; ++i) acc[1][b - 1][i] += p1[i] * s1_prev;
+                    }
+                    if (u == 1) loads(2 * b);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                s0 = bs * w0;
+                s1_prev = bs * w1;
+                if (b + 1 < NB) bs = read_bs(b + 1);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {  // chain of A tile 1; p0 is promoted meanwhile
+                    const bf16x8 f0 = e4m3x8_to_bf16(q[0], q[1]);
+                    const bf16x8 f1 = e4m3x8_to_bf16(q[2], q[3]);
+                    if (u < 3) q = b_piece(b, u + 1);
+                    else if (b + 1 < NB) q = b_piece(b + 1, 0);
+                    p1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Ab[1][2 * u], f0, u == 0 ? floatx16{0} : p1, 0, 0, 0);
+#pragma unroll
+                    for (int i = 4 * u; i < 4 * u + 2; ++i) acc[0][b][i] += p0[i] * s0;
+                    p1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Ab[1][2 * u + 1], f1, p1, 0, 0, 0);
+#pragma unroll
+                    for (int i = 4 * u + 2; i < 4 * u + 4; ++i) acc[0][b][i] += p0[i] * s0;
+                    if (u == 1) loads(2 * b + 1);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            acc[1][NB - 1] += p1 * s1_prev;
+            return;
+        }
         if constexpr (UE8M0) {
             // exponent bytes of the three scales; opsel 0 = byte 0 of the scale register
             const int e0 = (int)((__float_as_uint(w0) >> 23) & 255u);
@@ -411,7 +515,6 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
         acc[1][NB > 0 ? NB - 1 : 0] += p1 * s1_prev;
     };
 
-    PHASE_TIMING_BEGIN();
     issue_scales(0, 0, half_tile, 0);
 #pragma unroll
     for (int i = 4; i < 8; ++i) issue_load(0, i, 0);
@@ -488,12 +591,21 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
         float* s_amax = reinterpret_cast<float*>(s_stage);                      // [4 row groups][256 pairs]
         constexpr int CODE_ROW = GROUP + 16;                                    // bytes per pair row of codes
         uint8_t* s_codes = s_stage + 4 * TILE_PAIRS * sizeof(float);            // [256 pairs][CODE_ROW]
-        // FIX: marks staged like the codes, and three more per-pair statistics
-        uint8_t* s_marks = s_codes + TILE_PAIRS * CODE_ROW;
-        float* s_sumsq = reinterpret_cast<float*>(s_marks + TILE_PAIRS * CODE_ROW);
+        // FIX: three more per-pair statistics, the marks of every lane's 16 elements as bit masks, the pairs'
+        // scales and the list of pairs that hold a marked element
+        float* s_sumsq = reinterpret_cast<float*>(s_codes + TILE_PAIRS * CODE_ROW);
         float* s_umax = s_sumsq + 4 * TILE_PAIRS;
         float* s_sgmax = s_umax + 4 * TILE_PAIRS;
-        static_assert(16 * TILE_PAIRS * sizeof(float) + 2 * TILE_PAIRS * CODE_ROW <= 2 * STAGE_BYTES, "epilogue LDS");
+        uint16_t* s_near = reinterpret_cast<uint16_t*>(s_sgmax + 4 * TILE_PAIRS);  // [256 pairs][4 row groups][2 halves]
+        uint16_t* s_cand = s_near + 8 * TILE_PAIRS;
+        float* s_scale = reinterpret_cast<float*>(s_cand + 8 * TILE_PAIRS);      // [256 pairs]
+        int* s_list = reinterpret_cast<int*>(s_scale + TILE_PAIRS);              // [256]
+        int* s_count = s_list + TILE_PAIRS;
+        static_assert(18 * TILE_PAIRS * sizeof(float) + 16 * TILE_PAIRS * sizeof(uint16_t) + TILE_PAIRS * CODE_ROW + 16 <=
+                          2 * STAGE_BYTES, "epilogue LDS");
+        if constexpr (FIX) {
+            if (threadIdx.x == 0) *s_count = 0;
+        }
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
             float m = 0.f, sumsq = 0.f, umax = 0.f, sgmax = 0.f;
@@ -528,6 +640,8 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
             const float m = fmaxf(fmaxf(s_amax[pl], s_amax[TILE_PAIRS + pl]),
                                   fmaxf(s_amax[2 * TILE_PAIRS + pl], s_amax[3 * TILE_PAIRS + pl]));
             const float scale = group_scale(m, UE8M0);
+            // (v * (1 / scale) is within an ulp of v / scale, which the exact forms use: they can differ only
+            // where fp32 itself does not decide the code)
             const float inv_scale = 1.f / scale;
             float err = 0.f, dh_max = 0.f;
             bool uncertain = false;
@@ -542,35 +656,118 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
                 dh_max = (1.1f * umax + sgmax) * err;
                 uncertain = !UE8M0 || group_scale(m + dh_max, true) != group_scale(m - dh_max, true);
             }
+            uint32_t near_bits = 0, cand_bits = 0;
 #pragma unroll
             for (int qd = 0; qd < 4; ++qd) {
                 float q[4];
-                uint32_t marks = 0;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     float v = acc[0][b][4 * qd + r];
                     if constexpr (FIX) {
                         const float sg = silu(v);
                         v = sg * acc[1][b][4 * qd + r];
-                        marks |= requant_marks(v, sg, acc[1][b][4 * qd + r], scale, fmaxf(m, AMAX_FLOOR), err, dh_max,
-                                               uncertain)
-                                 << (8 * r);
+                        const uint32_t marks = requant_marks(v, sg, acc[1][b][4 * qd + r], scale, fmaxf(m, AMAX_FLOOR), err,
+                                                             dh_max, uncertain, v_min);
+                        near_bits |= (marks & MARK_NEAR ? 1u : 0u) << (4 * qd + r);
+                        cand_bits |= (marks & MARK_CANDIDATE ? 1u : 0u) << (4 * qd + r);
                     }
                     q[r] = fminf(fmaxf(v * inv_scale, -E4M3_MAX), E4M3_MAX);
                 }
                 int packed = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], 0, false);
                 packed = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], packed, true);
                 *reinterpret_cast<int*>(s_codes + pl * CODE_ROW + rg * 32 + 8 * qd + 4 * half) = packed;
-                if constexpr (FIX)
-                    *reinterpret_cast<uint32_t*>(s_marks + pl * CODE_ROW + rg * 32 + 8 * qd + 4 * half) = marks;
             }
-            if (rg == 0 && half == 0 && pl < cnt) {
+            if constexpr (FIX) {
+                s_near[pl * 8 + rg * 2 + half] = (uint16_t)near_bits;
+                s_cand[pl * 8 + rg * 2 + half] = (uint16_t)cand_bits;
+                if (rg == 0 && half == 0) s_scale[pl] = scale;
+            } else if (rg == 0 && half == 0 && pl < cnt) {
                 const size_t pos = (size_t)begin + pl;
                 h_s[pos * (inter / GROUP) + rb] = scale;
                 hs_t[(size_t)rb * scale_stride + pos] = scale;
             }
         }
         __syncthreads();
+        if constexpr (FIX) {
+            // Exact requantisation of the marked elements. The pairs that hold one are listed; the wavefronts take
+            // them in turn and recompute, as fp32 products of the codes summed in fp64 (the dot product itself
+            // to fp32 accuracy), first the elements that may be the pair's maximum over these 128 columns, which
+            // fixes the scale, then the marked elements, whose codes replace the staged ones. A recomputed element
+            // reads its activation row and its two weight rows (3 K bytes) once more, the weight rows from the L2
+            // this workgroup has just streamed them through.
+            if (threadIdx.x < TILE_PAIRS) {
+                const int pl = threadIdx.x;
+                const intx4 nm = *reinterpret_cast<const intx4*>(s_near + pl * 8);
+                if (pl < cnt && (nm[0] | nm[1] | nm[2] | nm[3]) != 0) s_list[atomicAdd(s_count, 1)] = pl;
+            }
+            __syncthreads();
+            const int n_list = *s_count;
+            const int n_chunks = K / 16;
+            for (int it = wave; it < n_list; it += 8) {
+                const int pl = __builtin_amdgcn_readfirstlane(s_list[it]);
+                const size_t pos = (size_t)begin + pl;
+                const uint8_t* x_row = a_q + (size_t)(sorted_pairs[pos] / top_k) * K;
+                const float* xs = as_t + pos;  // [kb * scale_stride]
+                const uint8_t* gate_rows = w_q + ((size_t)e * n_rows + rb * GROUP) * K;
+                auto exact_h = [&](int col) {  // h of column col of the group (every lane returns the same value)
+                    const uint8_t* gate_row = gate_rows + (size_t)col * K;
+                    const uint8_t* up_row = gate_row + (size_t)inter * K;
+                    double g = 0.0, u = 0.0;
+                    for (int c0 = 0; c0 < n_chunks; c0 += 256) {
+                        intx4 xq[4], wg[4], wu[4];
+                        float sg[4], su[4];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const int c = c0 + 64 * j + lane;
+                            xq[j] = wg[j] = wu[j] = intx4{0, 0, 0, 0};
+                            sg[j] = su[j] = 0.f;
+                            if (c < n_chunks) {
+                                xq[j] = *reinterpret_cast<const intx4*>(x_row + 16 * c);
+                                wg[j] = *reinterpret_cast<const intx4*>(gate_row + 16 * c);
+                                wu[j] = *reinterpret_cast<const intx4*>(up_row + 16 * c);
+                                const float x_scale = xs[(size_t)(c >> 3) * scale_stride];
+                                sg[j] = x_scale * ws0[c >> 3];
+                                su[j] = x_scale * ws1[c >> 3];
+                            }
+                        }
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            g += (double)(dot16(xq[j], wg[j]) * sg[j]);
+                            u += (double)(dot16(xq[j], wu[j]) * su[j]);
+                        }
+                    }
+                    const float gf = (float)wave_sum(g);
+                    const float uf = (float)wave_sum(u);
+                    return gf / (1.f + expf(-gf)) * uf;
+                };
+                auto column_of = [&](int part, int bit) { return (part >> 1) * 32 + 8 * (bit >> 2) + 4 * (part & 1) + (bit & 3); };
+                float scale = s_scale[pl];
+                float amax = 0.f;
+                bool any_candidate = false;
+                for (int part = 0; part < 8; ++part) {
+                    for (uint32_t cm = __builtin_amdgcn_readfirstlane((uint32_t)s_cand[pl * 8 + part]); cm != 0; cm &= cm - 1) {
+                        amax = fmaxf(amax, fabsf(exact_h(column_of(part, __builtin_ctz(cm)))));
+                        any_candidate = true;
+                    }
+                }
+                if (any_candidate) scale = group_scale(amax, UE8M0);
+                for (int part = 0; part < 8; ++part) {
+                    for (uint32_t nm = __builtin_amdgcn_readfirstlane((uint32_t)s_near[pl * 8 + part]); nm != 0; nm &= nm - 1) {
+                        const int col = column_of(part, __builtin_ctz(nm));
+                        const float v = fminf(fmaxf(exact_h(col) / scale, -E4M3_MAX), E4M3_MAX);
+                        const int code = __builtin_amdgcn_cvt_pk_fp8_f32(v, v, 0, false);
+                        if (lane == 0) s_codes[pl * CODE_ROW + col] = (uint8_t)(code & 0xff);
+                    }
+                }
+                if (lane == 0) s_scale[pl] = scale;
+            }
+            __syncthreads();
+            if (threadIdx.x < cnt) {
+                const size_t pos = (size_t)begin + threadIdx.x;
+                h_s[pos * (inter / GROUP) + rb] = s_scale[threadIdx.x];
+                hs_t[(size_t)rb * scale_stride + pos] = s_scale[threadIdx.x];
+            }
+        }
         // 8 lanes write the 128 codes of one pair: 8 pairs per instruction, 4 instructions per wavefront
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
@@ -579,9 +776,6 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
                 const size_t at = ((size_t)begin + pl) * inter + rb * GROUP + (lane & 7) * 16;
                 *reinterpret_cast<intx4*>(h_q + at) =
                     *reinterpret_cast<const intx4*>(s_codes + pl * CODE_ROW + (lane & 7) * 16);
-                if constexpr (FIX)
-                    *reinterpret_cast<intx4*>(h_marks + at) =
-                        *reinterpret_cast<const intx4*>(s_marks + pl * CODE_ROW + (lane & 7) * 16);
             }
         }
     } else {
@@ -672,15 +866,15 @@ extern "C" void moe_tiled_prepare_launcher(int* tile_start, float* xs_t, const f
                                                                     scale_stride, hidden / GROUP, top_k);
 }
 
-// h_marks / band_config (internal to the library): marks of the exact requantisation for
-// moe_requant_fix_launcher, [pairs, inter] bytes, or null; bits 10-11 of band_config scale the band.
-extern "C" void moe_gate_up_tiled_marked_launcher(void* h_q, float* h_s, float* hs_t, void* h_marks,
-                                                  const void* x_q, const float* xs_t, const void* w13_q,
-                                                  const float* w13_s, const int* sorted_pairs,
-                                                  const int* expert_offsets, const int* tile_start, int tokens,
-                                                  int hidden, int inter, int n_experts, int top_k,
-                                                  int scale_stride, int ue8m0, int band_config,
-                                                  hipStream_t stream) {
+// requant_config: the CONFIG_*_REQUANT, band and significance bits of the layer's config (moe_common.hpp):
+// neither requant bit: e4m3 matrix core, the marked elements repaired in the epilogue; CONFIG_EXACT_REQUANT: bf16
+// matrix core; CONFIG_APPROX_REQUANT: e4m3 matrix core, codes as they come.
+extern "C" void moe_gate_up_tiled_launcher(void* h_q, float* h_s, float* hs_t, const void* x_q,
+                                           const float* xs_t, const void* w13_q, const float* w13_s,
+                                           const int* sorted_pairs, const int* expert_offsets,
+                                           const int* tile_start, int tokens, int hidden, int inter,
+                                           int n_experts, int top_k, int scale_stride, int ue8m0,
+                                           int requant_config, hipStream_t stream) {
     if (tokens <= 0) return;
     if (hidden % GROUP != 0 || inter % GROUP != 0 || hidden <= 0 || inter <= 0 ||
         (unsigned long long)tokens * hidden >= (1ull << 32)) {  // 32-bit activation offsets
@@ -689,24 +883,16 @@ extern "C" void moe_gate_up_tiled_marked_launcher(void* h_q, float* h_s, float* 
     }
     const int max_tiles = (tokens * top_k) / TILE_PAIRS + n_experts;
     const dim3 grid(tiled_grid(inter / GROUP, max_tiles));
-    const auto kernel = h_marks ? (ue8m0 ? moe_tiled_gemm_kernel<true, true, true> : moe_tiled_gemm_kernel<true, false, true>)
-                                : (ue8m0 ? moe_tiled_gemm_kernel<true, true, false> : moe_tiled_gemm_kernel<true, false, false>);
+    const bool bf16_core = (requant_config & CONFIG_EXACT_REQUANT) != 0 && !(requant_config & CONFIG_APPROX_REQUANT);
+    const bool repair = !bf16_core && !(requant_config & CONFIG_APPROX_REQUANT);
+    const auto kernel = bf16_core ? (ue8m0 ? moe_tiled_gemm_kernel<true, true, false, true> : moe_tiled_gemm_kernel<true, false, false, true>)
+                        : repair  ? (ue8m0 ? moe_tiled_gemm_kernel<true, true, true> : moe_tiled_gemm_kernel<true, false, true>)
+                                  : (ue8m0 ? moe_tiled_gemm_kernel<true, true, false> : moe_tiled_gemm_kernel<true, false, false>);
     kernel<<<grid, 512, 0, stream>>>(
         static_cast<const uint8_t*>(w13_q), w13_s, static_cast<const uint8_t*>(x_q), xs_t, sorted_pairs,
         expert_offsets, tile_start, static_cast<uint8_t*>(h_q), h_s, hs_t, nullptr, nullptr, hidden, 2 * inter,
-        inter, top_k, n_experts, scale_stride, static_cast<uint8_t*>(h_marks),
-        requant_error_coefficient(band_config));
-}
-
-extern "C" void moe_gate_up_tiled_launcher(void* h_q, float* h_s, float* hs_t, const void* x_q,
-                                           const float* xs_t, const void* w13_q, const float* w13_s,
-                                           const int* sorted_pairs, const int* expert_offsets,
-                                           const int* tile_start, int tokens, int hidden, int inter,
-                                           int n_experts, int top_k, int scale_stride, int ue8m0,
-                                           hipStream_t stream) {
-    moe_gate_up_tiled_marked_launcher(h_q, h_s, hs_t, nullptr, x_q, xs_t, w13_q, w13_s, sorted_pairs,
-                                      expert_offsets, tile_start, tokens, hidden, inter, n_experts, top_k,
-                                      scale_stride, ue8m0, 0, stream);
+        inter, top_k, n_experts, scale_stride, requant_error_coefficient(requant_config),
+        requant_min_magnitude(requant_config));
 }
 
 // y [pairs, hidden] as fp16 of y / y_scale (the buffer's first pairs * hidden * 2 bytes), y_scale
@@ -728,5 +914,5 @@ extern "C" void moe_down_tiled_launcher(void* y, float* y_scale, const void* h_q
     kernel<<<grid, 512, 0, stream>>>(
         static_cast<const uint8_t*>(w2_q), w2_s, static_cast<const uint8_t*>(h_q), hs_t, nullptr,
         expert_offsets, tile_start, nullptr, nullptr, nullptr, static_cast<float*>(y), y_scale, inter, hidden,
-        inter, top_k, n_experts, scale_stride, nullptr, 0.f);
+        inter, top_k, n_experts, scale_stride, 0.f, 0.f);
 }

@@ -24,19 +24,6 @@ extern "C" void moe_down_launcher(float* y, const void* h_q, const float* h_s, c
                                   const float* w2_s, const int* expert_offsets, int tokens, int hidden,
                                   int inter, int n_experts, int top_k, int config, hipStream_t stream);
 
-extern "C" void moe_gate_up_tiled_marked_launcher(void* h_q, float* h_s, float* hs_t, void* h_marks,
-                                                  const void* x_q, const float* xs_t, const void* w13_q,
-                                                  const float* w13_s, const int* sorted_pairs,
-                                                  const int* expert_offsets, const int* tile_start, int tokens,
-                                                  int hidden, int inter, int n_experts, int top_k,
-                                                  int scale_stride, int ue8m0, int band_config,
-                                                  hipStream_t stream);
-extern "C" void moe_requant_fix_launcher(void* h_q, float* h_s, float* hs_t, const void* h_marks,
-                                         const void* x_q, const float* x_s, const void* w13_q,
-                                         const float* w13_s, const int* sorted_pairs,
-                                         const int* expert_offsets, int tokens, int hidden, int inter,
-                                         int n_experts, int top_k, int scale_stride, int ue8m0,
-                                         hipStream_t stream);
 extern "C" void moe_tiled_prepare_launcher(int* tile_start, float* xs_t, const float* x_s,
                                            const int* sorted_pairs, const int* expert_offsets,
                                            int tokens, int hidden, int n_experts, int top_k,
@@ -46,7 +33,7 @@ extern "C" void moe_gate_up_tiled_launcher(void* h_q, float* h_s, float* hs_t, c
                                            const int* sorted_pairs, const int* expert_offsets,
                                            const int* tile_start, int tokens, int hidden, int inter,
                                            int n_experts, int top_k, int scale_stride, int ue8m0,
-                                           hipStream_t stream);
+                                           int requant_config, hipStream_t stream);
 extern "C" void moe_down_tiled_launcher(void* y, float* y_scale, const void* h_q, const float* hs_t,
                                         const void* w2_q, const float* w2_s, const int* expert_offsets,
                                         const int* tile_start, int tokens, int hidden, int inter,
@@ -191,26 +178,27 @@ extern "C" size_t moe_fp8_workspace_bytes(int tokens, int hidden, int inter, int
 }
 
 // Byte offsets of the intermediate buffers inside the workspace, in the order
-// ids, weights, expert_offsets, sorted_pairs, pair_pos, x_q, x_s, h_q, h_s, y, h_marks, y_scale
-// (for checkers that compare the stages against a reference).
-extern "C" void moe_fp8_workspace_layout(size_t* offsets12, int tokens, int hidden, int inter,
-                                         int n_experts, int top_k) {
+// ids, weights, expert_offsets, sorted_pairs, pair_pos, x_q, x_s, h_q, h_s, y, y_scale
+// (for checkers that compare the stages against a reference). Writes min(n_offsets, 11) entries and returns
+// the number of entries the layout has, so that a caller built against another version of this list notices.
+extern "C" int moe_fp8_workspace_layout(size_t* offsets, int n_offsets, int tokens, int hidden, int inter,
+                                        int n_experts, int top_k) {
     char* base = reinterpret_cast<char*>(uintptr_t{4096});
     const moe::Workspace w = moe::carve_workspace(base, tokens, hidden, inter, n_experts, top_k);
-    const void* ptrs[12] = {w.ids, w.weights, w.expert_offsets, w.sorted_pairs, w.pair_pos, w.x_q,
-                            w.x_s, w.h_q,     w.h_s,            w.y,            w.h_marks,  w.y_scale};
-    for (int i = 0; i < 12; ++i) offsets12[i] = static_cast<const char*>(ptrs[i]) - base;
+    const void* ptrs[11] = {w.ids, w.weights, w.expert_offsets, w.sorted_pairs, w.pair_pos, w.x_q,
+                            w.x_s, w.h_q,     w.h_s,            w.y,            w.y_scale};
+    for (int i = 0; i < 11 && i < n_offsets; ++i) offsets[i] = static_cast<const char*>(ptrs[i]) - base;
+    return 11;
 }
 
 namespace {
 
-// How the expert GEMMs of one group of experts run: LDS-tiled or weight-streaming form, with or without the
-// exact requantisation pass. Resolved, and checked against what the chosen kernels support, before the first
-// launch of a layer, so that a shape one stage rejects launches nothing at all.
+// How the expert GEMMs of one group of experts run: LDS-tiled or weight-streaming form. Resolved, and checked
+// against what the chosen kernels support, before the first launch of a layer, so that a shape one stage rejects
+// launches nothing at all.
 struct GemmPlan {
     bool ok;
     bool tiled;
-    bool exact;
 };
 
 GemmPlan plan_expert_gemms(int tokens, int hidden, int inter, int n_experts, int top_k, int config) {
@@ -222,11 +210,6 @@ GemmPlan plan_expert_gemms(int tokens, int hidden, int inter, int n_experts, int
     GemmPlan plan{};
     plan.tiled = form == 16 || (form == 0 && (long)tokens * top_k > 32L * n_experts && tiled_ok);
     plan.ok = !plan.tiled || tiled_ok;
-    // The streaming gate/up GEMM is exact by itself (bf16 matrix core; e4m3 on request). The tiled one runs on
-    // the e4m3 matrix core and is followed by the pass that recomputes marked elements only on request: with
-    // thousands of pairs per expert that pass re-reads two weight rows for every few dozen elements of h.
-    plan.exact = plan.tiled && (config & CONFIG_EXACT_REQUANT) != 0 && !(config & CONFIG_APPROX_REQUANT);
-    if (plan.exact && hidden > 16384) plan.ok = false;
     return plan;
 }
 
@@ -237,20 +220,16 @@ void run_expert_gemms(const moe::Workspace& w, const GemmPlan& plan, const void*
                       int n_experts, int top_k, int config, hipStream_t stream) {
     const int ue8m0 = config & CONFIG_UE8M0;  // power-of-two block scales, see moe_fp8_launcher
     const int order = config & CONFIG_LAST_EXPERT_FIRST;
-    const int band = config & CONFIG_BAND_MASK;
+    int requant = config & CONFIG_REQUANT_BITS;
+    if (!(requant & CONFIG_SIGNIF_MASK)) requant |= default_requant_significance(inter, top_k) << CONFIG_SIGNIF_SHIFT;
     const int approx = config & CONFIG_APPROX_REQUANT;
     config &= ~(CONFIG_UE8M0 | CONFIG_LAST_EXPERT_FIRST | CONFIG_REQUANT_BITS);
-    uint8_t* marks = plan.exact ? w.h_marks : nullptr;
     if (plan.tiled) {
         moe_tiled_prepare_launcher(w.tile_start, w.xs_t, w.x_s, w.sorted_pairs, w.expert_offsets, tokens,
                                    hidden, n_experts, top_k, w.scale_stride, stream);
-        moe_gate_up_tiled_marked_launcher(w.h_q, w.h_s, w.hs_t, marks, w.x_q, w.xs_t, w13_q, w13_s,
-                                          w.sorted_pairs, w.expert_offsets, w.tile_start, tokens, hidden, inter,
-                                          n_experts, top_k, w.scale_stride, ue8m0, band, stream);
-        if (marks)
-            moe_requant_fix_launcher(w.h_q, w.h_s, w.hs_t, marks, w.x_q, w.x_s, w13_q, w13_s, w.sorted_pairs,
-                                     w.expert_offsets, tokens, hidden, inter, n_experts, top_k, w.scale_stride,
-                                     ue8m0, stream);
+        moe_gate_up_tiled_launcher(w.h_q, w.h_s, w.hs_t, w.x_q, w.xs_t, w13_q, w13_s, w.sorted_pairs,
+                                   w.expert_offsets, w.tile_start, tokens, hidden, inter, n_experts, top_k,
+                                   w.scale_stride, ue8m0, requant, stream);
         moe_down_tiled_launcher(w.y, w.y_scale, w.h_q, w.hs_t, w2_q, w2_s, w.expert_offsets, w.tile_start, tokens,
                                 hidden, inter, n_experts, top_k, w.scale_stride, ue8m0, stream);
     } else {

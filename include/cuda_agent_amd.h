@@ -382,15 +382,14 @@ void moe_combine_launcher(void* out, const float* y, const float* weights, const
 size_t moe_fp8_workspace_bytes(int tokens, int hidden, int inter, int n_experts, int top_k);
 
 /* Byte offsets, inside that workspace, of ids, weights, expert_offsets, sorted_pairs, pair_pos,
- * x_q, x_s, h_q, h_s, y, h_marks, y_scale (in this order), for checkers that inspect the stages.
+ * x_q, x_s, h_q, h_s, y, y_scale (in this order), for checkers that inspect the stages. Writes
+ * min(n_offsets, 11) entries and returns the number of fields the layout has (11), so that a caller
+ * built against another version of the list can tell.
  * y [tokens*top_k, hidden]: fp32 rows when the layer ran the weight-streaming GEMMs; when it ran the
  * LDS-tiled ones (moe_fp8_uses_tiled_gemms), fp16 rows in the first half of the buffer, to be
- * multiplied by y_scale [tokens*top_k, hidden/256] (one power of two per row and run of 256 columns).
- * h_marks [tokens*top_k, inter] bytes: bit 0 = the element was within the matrix core's error of an
- * e4m3 rounding boundary, bit 1 = it may have been its group's maximum (written only when the exact
- * requantisation pass runs, see moe_fp8_launcher). */
-void moe_fp8_workspace_layout(size_t* offsets12, int tokens, int hidden, int inter, int n_experts,
-                              int top_k);
+ * multiplied by y_scale [tokens*top_k, hidden/256] (one power of two per row and run of 256 columns). */
+int moe_fp8_workspace_layout(size_t* offsets, int n_offsets, int tokens, int hidden, int inter,
+                             int n_experts, int top_k);
 
 /* 1 if moe_fp8_launcher runs these sizes and this config on the LDS-tiled GEMMs, 0 if on the
  * weight-streaming ones, -1 if it rejects them. */
@@ -406,14 +405,19 @@ int moe_fp8_uses_tiled_gemms(int tokens, int hidden, int inter, int n_experts, i
  * every block scale is a power of two (UE8M0). w13_s and w2_s must then hold powers of two; x and
  * the intermediate are quantised with scale = the smallest power of two >= max(amax, 1e-12)/448,
  * and the tiled GEMMs apply the scales inside the MFMA.
- * +256 / +512: exact requantisation of the intermediate on / off. The e4m3 matrix core sums a
+ * +256 / +512: how the intermediate h = silu(g) * u is requantised. The e4m3 matrix core sums a
  * 128-block with about 16 significant bits, so about one code of h in a thousand would differ by one
- * step from an fp32 evaluation; with the pass on, the elements within that error of a rounding
- * boundary and the candidates for a group's maximum are recomputed as fp32 dot products between the
- * gate/up and the down stage. Default (neither bit): on with the streaming GEMMs (a few percent of a
- * decode step), off with the tiled ones (the pass re-reads two weight rows per recomputed element,
- * which for thousands of pairs per expert costs more than the layer). +1024 / +2048 / +3072: the
- * band that selects the elements is half / twice / four times as wide. */
+ * step from an fp32 evaluation, and one step on an element near its group's maximum moves single
+ * outputs by up to 3 % of their rms. The streaming gate/up GEMM therefore runs on the bf16 matrix core
+ * (exact sums, same time: it is bound by the weight stream); +512 puts it on the e4m3 one. The tiled
+ * gate/up GEMM by default stays on the e4m3 matrix core and recomputes, in its epilogue, the elements
+ * in the two highest binades of their group's range (at least 128 of 448 code units) that lie within
+ * the matrix core's error of a rounding boundary, together with the candidates for the maximum of
+ * those groups, as plain dot products: codes of large elements as an fp32 evaluation gives them,
+ * small ones (a code step of at most 8/448 of the group's maximum) as the matrix core rounds them.
+ * +256: the tiled gate/up GEMM on the bf16 matrix core instead: every code exact, twice the
+ * matrix-core time. +512: e4m3 matrix core, no repair. +1024 / +2048 / +3072: the band is half /
+ * twice / four times as wide. +4096*s (s = 1..8): repair elements of at least 2^s code units. */
 void moe_fp8_launcher(void* out, const void* x, const float* logits, const void* w13_q,
                       const float* w13_s, const void* w2_q, const float* w2_s, void* workspace,
                       size_t workspace_bytes, int tokens, int hidden, int inter, int n_experts,

@@ -17,12 +17,12 @@ import torch
 
 from oracle import moe
 
-from moe_checks import code_steps, oracle_down, settle_disputed_codes
+from moe_checks import code_steps, oracle_down, repaired_below, settle_disputed_codes
 
 pytestmark = pytest.mark.gpu
 TOL = 2e-2
-EXACT_REQUANT = 256   # config bit of the layer: the exact requantisation pass behind the tiled gate/up GEMM
-APPROX_REQUANT = 512  # config bit of the layer: the streaming gate/up GEMM on the e4m3 matrix core
+EXACT_REQUANT = 256   # config bit of the layer: the tiled gate/up GEMM on the bf16 matrix core (every code of h exact)
+APPROX_REQUANT = 512  # config bit of the layer: gate/up on the e4m3 matrix core, codes of h as they come
 
 
 def make_case(dev, T, H, I, E, seed, biased=None):
@@ -104,16 +104,21 @@ def test_activation_quantisation_bit_exact(capi, dev):
     assert torch.equal(q.cpu().view(torch.uint8), want_q.view(torch.uint8))
 
 
-def check_layer(capi, dev, T, H, I, E, k, seed, config=0, biased=None):
+def check_layer(capi, dev, T, H, I, E, k, seed, config=0, biased=None, requant='exact'):
     """Stage-wise parity: every stage is compared with the oracle's evaluation of that stage, the
     floating-point stages on the kernel's own output of the stage before; then the layer output end to end:
-    max |error| <= 2e-2 of the output rms. The requantised codes of h must equal the oracle's except where an
-    fp32 evaluation is itself undecided (settle_disputed_codes): a handful per million. (The e4m3 matrix core
-    alone, which sums a 128-block with about 16 significant bits, would put about one code in a thousand on
-    the other side of a rounding boundary and move isolated outputs by 2-4 % of the rms; the streaming gate/up
-    GEMM therefore runs on the bf16 matrix core and the tiled one is followed by the exact requantisation
-    pass when config bit 256 asks for it, as every tiled case here does.)"""
-    config |= EXACT_REQUANT   # (only the tiled form looks at it)
+    max |error| <= 2e-2 of the output rms.
+    requant 'exact' (the streaming gate/up GEMM, which runs on the bf16 matrix core, and the tiled one with
+    config bit 256, likewise): the requantised codes of h must equal the oracle's except where an fp32
+    evaluation is itself undecided (settle_disputed_codes): a handful per million.
+    requant 'repaired' (the tiled gate/up GEMM as the layer runs it by default: e4m3 matrix core, which sums a
+    128-block with about 16 significant bits and so puts about one code in a thousand on the other side of a
+    rounding boundary, and an epilogue that recomputes the elements of at least repaired_below(I, k) of 448 code
+    units that lie near a boundary): codes above that as in 'exact'; smaller ones may be a step off, and what that does to
+    the output counts towards the end-to-end bound."""
+    exact_codes = requant == 'exact'
+    if exact_codes:
+        config |= EXACT_REQUANT   # (only the tiled form looks at it)
     x, logits, w, dts = make_case(dev, T, H, I, E, seed, biased)
     w13_q, w13_s, w2_q, w2_s = w
     ref, mid = moe.moe_forward(x, logits, *w, top_k=k, out_dtype=torch.float32, return_intermediates=True)
@@ -130,10 +135,11 @@ def check_layer(capi, dev, T, H, I, E, k, seed, config=0, biased=None):
     pos = pos.long()
     hq = views['h_q'].cpu()[pos].reshape(T, k, I)
     hs = views['h_s'].cpu()[pos].reshape(T, k, I // 128)
-    torch.testing.assert_close(hs, mid['h_s'], rtol=1e-5, atol=0)
+    torch.testing.assert_close(hs, mid['h_s'], rtol=1e-5 if exact_codes else 3e-4, atol=0)
     code_diff = code_steps(hq, mid['h_q'])
-    assert (code_diff > 0).float().mean().item() < 2e-4
-    assert not (code_diff > 1).any()                         # never more than one code step
+    assert (code_diff > 0).float().mean().item() < (2e-4 if exact_codes else 4e-3)
+    if exact_codes:
+        assert not (code_diff > 1).any()                     # never more than one code step
     # down projection, on the kernel's own h (the tiled form stores y with 11 significant bits relative to the
     # largest value of each run of 256 columns: up to 2.5e-3 of the rms)
     y = views['y'].cpu()[pos].reshape(T, k, H)
@@ -144,11 +150,12 @@ def check_layer(capi, dev, T, H, I, E, k, seed, config=0, biased=None):
         want += mid['weights'][:, j:j + 1] * y[:, j]
     assert moe.rel_rms_error(exact.cpu(), want) <= 1e-5
     # end to end
-    n_disputed, settled = settle_disputed_codes(hq, mid, w13_q, w13_s, w2_q, w2_s, k)
+    n_settled, settled = settle_disputed_codes(hq, mid, w13_q, w13_s, w2_q, w2_s, k,
+                                               small_below=0 if exact_codes else repaired_below(I, k))
     err, err_settled = moe.rel_rms_error(exact.cpu(), ref), moe.rel_rms_error(exact.cpu(), settled)
-    print(f'[moe] T={T} H={H} I={I} E={E} k={k} config={config}: {n_disputed} of {hq.numel()} h codes differ from '
-          f'the oracle (all undecided in fp32), end-to-end max error {err:.2e} of the output rms, '
-          f'{err_settled:.2e} with those codes settled')
+    print(f'[moe] T={T} H={H} I={I} E={E} k={k} config={config} ({requant}): {int((code_diff > 0).sum())} of {hq.numel()} h '
+          f'codes differ from the oracle, {n_settled} of them undecided in fp32; end-to-end max error {err:.2e} of the '
+          f'output rms raw, {err_settled:.2e} with the undecided codes settled')
     assert err_settled <= TOL
     out, _ = run_layer(capi, dts, k, config)
     assert torch.equal(out, exact.bfloat16())
@@ -160,21 +167,24 @@ def test_layer_small(capi, dev, config):
     check_layer(capi, dev, T=40, H=512, I=256, E=8, k=2, seed=41, config=config)
 
 
+@pytest.mark.parametrize('requant', ['exact', 'repaired'])
 @pytest.mark.parametrize('shape', [(300, 512, 256, 4, 2), (700, 256, 128, 2, 1), (520, 768, 384, 3, 3),
                                    (64, 256, 128, 4, 4)])
-def test_layer_tiled_gemms(capi, dev, shape):
+def test_layer_tiled_gemms(capi, dev, shape, requant):
     # config 16 forces the LDS-tiled GEMMs: full 256-pair tiles, ragged last tiles, experts with
-    # fewer pairs than one tile, several row tiles
+    # fewer pairs than one tile, several row tiles; gate/up on the bf16 matrix core ('exact') and on the e4m3
+    # matrix core with the repair of the large codes in its epilogue (the default)
     T, H, I, E, k = shape
-    check_layer(capi, dev, T=T, H=H, I=I, E=E, k=k, seed=50 + T, config=16)
+    check_layer(capi, dev, T=T, H=H, I=I, E=E, k=k, seed=50 + T, config=16, requant=requant)
 
 
 @pytest.mark.parametrize('seed', range(8))
 def test_tiled_and_streaming_forms_agree_on_random_shapes(capi, dev, seed):
     # Random sizes and routing skews: experts with no pairs, with a few, with several 256-pair tiles;
-    # 1 to 7 K blocks in either GEMM. The integer stages must be identical; the codes of h (tiled GEMMs + exact
-    # requantisation pass against the streaming GEMMs on the bf16 matrix core) may differ where fp32 itself is
-    # undecided; each output meets the end-to-end bound against the oracle with such codes settled.
+    # 1 to 7 K blocks in either GEMM. The integer stages must be identical; the codes of h (tiled gate/up GEMM
+    # against the streaming one, both on the bf16 matrix core) may differ where fp32 itself is undecided; each
+    # output, and that of the tiled form as it runs by default (e4m3 matrix core, large codes repaired), meets
+    # the end-to-end bound against the oracle with such codes settled.
     rng = torch.Generator().manual_seed(1000 + seed)
     pick = lambda xs: xs[int(torch.randint(len(xs), (1,), generator=rng))]
     H, I = pick([256, 512, 768]), pick([128, 256, 384, 896])
@@ -192,28 +202,37 @@ def test_tiled_and_streaming_forms_agree_on_random_shapes(capi, dev, seed):
     assert torch.isfinite(a).all() and torch.isfinite(b).all()
     ref, mid = moe.moe_forward(x, logits, *w, top_k=k, out_dtype=torch.float32, return_intermediates=True)
     pos = va['pair_pos'].cpu().long()
-    for got, views in ((a, va), (b, vb)):
+    c, vc = run_layer(capi, dts, k, 16, torch.float32)                   # tiled GEMMs as they run by default
+    for got, views, small in ((a, va, 0), (b, vb, 0), (c, vc, repaired_below(I, k))):
         hq = views['h_q'].cpu()[pos].reshape(T, k, I)
-        _, settled = settle_disputed_codes(hq, mid, *w, k)
+        _, settled = settle_disputed_codes(hq, mid, *w, k, small_below=small)
         assert moe.rel_rms_error(got.cpu(), settled) <= TOL
 
 
 def test_requantisation_on_the_e4m3_matrix_core_is_what_the_exact_forms_remove(capi, dev):
-    # The same layer three ways: streaming gate/up on the e4m3 matrix core (config bit 512), on the bf16 one
-    # (default), and tiled GEMMs without and with the exact pass. The e4m3 forms differ from the oracle in about
-    # one code of h in a thousand, the exact forms in none or a few per million.
+    # The same layer five ways: streaming gate/up on the e4m3 matrix core (config bit 512) and on the bf16 one
+    # (default); tiled gate/up on the e4m3 matrix core as it comes (512), with the repair of the large codes
+    # (default) and on the bf16 matrix core (256). The e4m3 forms differ from the oracle in about one code of h
+    # in a thousand, the bf16 forms in none or a few per million; the repaired form like the e4m3 one over all
+    # codes and like the bf16 ones over the codes above 128 of 448 units.
     T, H, I, E, k = 300, 512, 256, 4, 2
     x, logits, w, dts = make_case(dev, T, H, I, E, 350)
     _, mid = moe.moe_forward(x, logits, *w, top_k=k, out_dtype=torch.float32, return_intermediates=True)
-    rate = {}
-    for name, config in (('stream e4m3', 4 | APPROX_REQUANT), ('stream bf16', 4), ('tiled', 16),
-                         ('tiled exact', 16 | EXACT_REQUANT)):
+    table = torch.from_numpy(moe.e4m3_decode_table())
+    large = table[(mid['h_q'].view(torch.uint8) & 0x7f).long()] > repaired_below(I, k)
+    rate, rate_large = {}, {}
+    for name, config in (('stream e4m3', 4 | APPROX_REQUANT), ('stream bf16', 4), ('tiled e4m3', 16 | APPROX_REQUANT),
+                         ('tiled repaired', 16), ('tiled bf16', 16 | EXACT_REQUANT)):
         _, views = run_layer(capi, dts, k, config, torch.float32)
         hq = views['h_q'].cpu()[views['pair_pos'].cpu().long()].reshape(T, k, I)
-        rate[name] = (code_steps(hq, mid['h_q']) > 0).float().mean().item()
-    print('[moe] h codes that differ from the oracle:', {n: f'{r * 1e6:.0f} ppm' for n, r in rate.items()})
-    assert 3e-4 < rate['stream e4m3'] < 3e-3 and 3e-4 < rate['tiled'] < 3e-3
-    assert rate['stream bf16'] < 1e-4 and rate['tiled exact'] < 1e-4
+        differ = code_steps(hq, mid['h_q']) > 0
+        rate[name] = differ.float().mean().item()
+        rate_large[name] = (differ & large).float().sum().item() / large.float().sum().item()
+    print('[moe] h codes that differ from the oracle:', {n: f'{r * 1e6:.0f} ppm' for n, r in rate.items()},
+          f'among the codes above {repaired_below(I, k):.0f} units:', {n: f'{r * 1e6:.0f} ppm' for n, r in rate_large.items()})
+    assert 3e-4 < rate['stream e4m3'] < 3e-3 and 3e-4 < rate['tiled e4m3'] < 3e-3 and 3e-4 < rate['tiled repaired'] < 3e-3
+    assert rate['stream bf16'] < 1e-4 and rate['tiled bf16'] < 1e-4
+    assert rate_large['tiled e4m3'] > 2e-4 and rate_large['tiled repaired'] < 1e-4
 
 
 def test_tiled_path_is_chosen_for_many_pairs_per_expert(capi, dev):
@@ -352,11 +371,10 @@ def oracle_on_tokens(tokens, dts, ids, k):
     return ref, mid
 
 
-def check_sampled_tokens(tokens, dts, ids, pos, views, exact, k, exact_requant=True):
-    """The stage-wise and end-to-end bounds of check_layer for a sample of tokens of a full-size layer.
-    exact_requant False: the layer ran the tiled GEMMs without the exact requantisation pass, so about one h
-    code in a thousand is one step off and the end-to-end error is reported, and bounded by 3x the tolerance,
-    instead of by the tolerance."""
+def check_sampled_tokens(tokens, dts, ids, pos, views, exact, k, requant='exact'):
+    """The stage-wise and end-to-end bounds of check_layer for a sample of tokens of a full-size layer
+    (requant as there: 'exact' or 'repaired')."""
+    exact_codes = requant == 'exact'
     H, I = dts[0].shape[1], dts[2].shape[1] // 2
     ref, mid = oracle_on_tokens(tokens, dts, ids, k)
     w13_q, w13_s, w2_q, w2_s = mid['w']
@@ -365,10 +383,10 @@ def check_sampled_tokens(tokens, dts, ids, pos, views, exact, k, exact_requant=T
     n = len(tokens)
     hq = views['h_q'].view(torch.uint8)[rows].cpu().view(torch.float8_e4m3fn).reshape(n, k, I)
     hs = views['h_s'][rows].cpu().reshape(n, k, I // 128)
-    torch.testing.assert_close(hs, mid['h_s'], rtol=1e-5 if exact_requant else 1e-3, atol=0)
+    torch.testing.assert_close(hs, mid['h_s'], rtol=1e-5 if exact_codes else 3e-4, atol=0)
     code_diff = code_steps(hq, mid['h_q'])
     flips = (code_diff > 0).float().mean().item()
-    assert flips < (2e-4 if exact_requant else 3e-3)
+    assert flips < (2e-4 if exact_codes else 4e-3)
     # (on the e4m3 matrix core a value near zero, where the format's steps are 2^-9 of the scale, can be two
     # steps off: its error is absolute, about 1e-5 of the rms of the pre-activations)
     far = code_diff > 1
@@ -376,7 +394,7 @@ def check_sampled_tokens(tokens, dts, ids, pos, views, exact, k, exact_requant=T
         table = torch.from_numpy(moe.e4m3_decode_table())
         print(f'[moe] {int(far.sum())} of {hq.numel()} h codes more than one step off, at most {int(code_diff.max())} steps, '
               f'largest magnitude among them {table[(mid["h_q"].view(torch.uint8)[far] & 0x7f).long()].max().item()} of 448')
-    assert not far.any() if exact_requant else far.float().mean().item() < 1e-4
+    assert not far.any() if exact_codes else far.float().mean().item() < 1e-4
     y = views['y'][rows].cpu().reshape(n, k, H)
     local = dict(mid, ids=mid['local_ids'])
     assert moe.rel_rms_error(y, oracle_down(hq, hs, mid['local_ids'], w2_q, w2_s)) <= 3e-3
@@ -386,18 +404,13 @@ def check_sampled_tokens(tokens, dts, ids, pos, views, exact, k, exact_requant=T
     got = exact[tokens.to(exact.device)].cpu()
     assert moe.rel_rms_error(got, want) <= 1e-5
     err = moe.rel_rms_error(got, ref)
-    if exact_requant:
-        n_disputed, settled = settle_disputed_codes(hq, local, w13_q, w13_s, w2_q, w2_s, k)
-        err_settled = moe.rel_rms_error(got, settled)
-        print(f'[moe] {n} sampled tokens: {n_disputed} of {hq.numel()} h codes differ from the oracle (all undecided '
-              f'in fp32), end-to-end max error {err:.2e} of the output rms, {err_settled:.2e} with those settled')
-        assert err_settled <= TOL
-    else:
-        beyond = ((got - ref).abs() > TOL * ref.double().pow(2).mean().sqrt()).float().mean().item()
-        print(f'[moe] {n} sampled tokens, e4m3 matrix core without the exact pass: {flips * 1e3:.2f} per mille of h '
-              f'codes one step off, end-to-end max error {err:.2e} of the output rms, {beyond * 1e6:.0f} ppm of '
-              f'the outputs beyond {TOL}')
-        assert err <= 3 * TOL and beyond <= 1e-3
+    n_settled, settled = settle_disputed_codes(hq, local, w13_q, w13_s, w2_q, w2_s, k,
+                                               small_below=0 if exact_codes else repaired_below(I, k))
+    err_settled = moe.rel_rms_error(got, settled)
+    print(f'[moe] {n} sampled tokens ({requant}): {flips * 1e6:.0f} ppm of the h codes differ from the oracle, {n_settled} '
+          f'codes undecided in fp32; end-to-end max error {err:.2e} of the output rms raw, {err_settled:.2e} with the '
+          f'undecided codes settled')
+    assert err_settled <= TOL
     return err
 
 
@@ -406,14 +419,16 @@ def test_full_prefill_workload_properties(capi, dev):
     the activation codes against the oracle at full size. The floating-point stages and the end-to-end bound
     against the oracle on sampled tokens that sit in the first, a middle and the ragged last 256-pair tile of
     the most loaded expert and in the first and last pair of four lightly loaded experts: for the layer as it
-    runs by default at this size (tiled GEMMs on the e4m3 matrix core: the deviation is printed and bounded by
-    3x the tolerance), and with the exact requantisation pass (the stated tolerance). The whole output against
-    the weight-streaming form of the layer (separately written kernels); all outputs finite; the bf16 output
-    equal to the rounding of the fp32 one."""
+    runs by default at this size (tiled GEMMs, gate/up on the e4m3 matrix core with the large codes repaired)
+    and with gate/up on the bf16 matrix core (config bit 256: every code exact), both to the stated tolerance.
+    The whole output of the default form against that of the exact one, again to the tolerance, and the exact
+    one against the weight-streaming form of the layer (separately written kernels); all outputs finite; the
+    bf16 output equal to the rounding of the fp32 one."""
     T, H, I, E, k = 8192, 7168, 2048, 256, 8
     dts = full_size_layer(dev, T, 20254, n_biased=16)
     x, logits = dts[0], dts[1]
-    exact, views = run_layer(capi, dts, k, 0, torch.float32)       # config 0 must take the tiled GEMMs
+    default, views = run_layer(capi, dts, k, 0, torch.float32)       # config 0 must take the tiled GEMMs
+    assert capi.library().moe_fp8_uses_tiled_gemms(T, H, I, E, k, 0) == 1
     ids, weights = moe.route(logits.cpu(), k)
     assert torch.equal(views['ids'].cpu(), ids)
     torch.testing.assert_close(views['weights'].cpu(), weights, rtol=1e-6, atol=1e-7)
@@ -423,7 +438,7 @@ def test_full_prefill_workload_properties(capi, dev):
     x_q, x_s = moe.quantize_groups(x.cpu().float())
     assert torch.equal(views['x_q'].cpu().view(torch.uint8), x_q.view(torch.uint8))
     assert torch.equal(views['x_s'].cpu(), x_s)
-    assert torch.isfinite(exact).all()
+    assert torch.isfinite(default).all()
 
     counts = (off[1:] - off[:-1]).long()
     hot = int(counts.argmax())
@@ -439,43 +454,46 @@ def test_full_prefill_workload_properties(capi, dev):
     more = torch.randperm(T, generator=torch.Generator().manual_seed(4))[:16 - len(tokens)].tolist()
     tokens = sorted(set(tokens) | set(more))
     assert len(tokens) >= 12
-    check_sampled_tokens(tokens, dts, ids, pos, views, exact, k, exact_requant=False)
+    check_sampled_tokens(tokens, dts, ids, pos, views, default, k, requant='repaired')
     out, _ = run_layer(capi, dts, k, 0)
-    assert torch.equal(out, exact.bfloat16())
+    assert torch.equal(out, default.bfloat16())
+    hq_default = views['h_q'].view(torch.uint8).clone()
     del out, views
 
-    # the same tiles with the exact requantisation pass behind the gate/up GEMM: the stated tolerance
-    fixed, views = run_layer(capi, dts, k, EXACT_REQUANT, torch.float32)
-    assert torch.isfinite(fixed).all()
-    check_sampled_tokens(tokens, dts, ids, pos, views, fixed, k)
-    marks = views['h_marks']
-    print(f'[moe] exact requantisation at full size: {(marks & 1).float().mean().item() * 100:.2f} % of the elements '
-          f'of h recomputed for their code, {((marks >> 1) & 1).float().mean().item() * 100:.2f} % as candidates '
-          f'for the maximum of their group')
-    hq_fixed = views['h_q'].clone()
-    del views, marks
-    # what leaving the pass out (the default at this size) does to the whole output
-    rms = fixed.double().pow(2).mean().sqrt()
-    diff = (exact - fixed).abs()
-    beyond = (diff > TOL * rms).float().mean().item()
-    print(f'[moe] tiled GEMMs without against with the exact pass at full size: rms difference '
-          f'{(diff.double().pow(2).mean().sqrt() / rms).item():.2e} of the output rms, max '
-          f'{(diff.max().double() / rms).item():.2e}, {beyond * 1e6:.2f} ppm of the outputs beyond {TOL}')
-    assert (diff.max().double() / rms).item() <= 3 * TOL and beyond <= 1e-4
-    del exact
+    # gate/up on the bf16 matrix core: every code of h as an fp32 evaluation gives it
+    exact, views = run_layer(capi, dts, k, EXACT_REQUANT, torch.float32)
+    assert torch.isfinite(exact).all()
+    check_sampled_tokens(tokens, dts, ids, pos, views, exact, k)
+    hq_exact = views['h_q'].view(torch.uint8).clone()
+    del views
+    # the default form against it over the whole output
+    differ = hq_default != hq_exact
+    large = (hq_exact & 0x7f) > 0x70                                  # magnitude above 128 of 448 units
+    print(f'[moe] h codes of the default form that differ from the exact one at full size: '
+          f'{differ.float().mean().item() * 1e6:.0f} ppm of all, '
+          f'{(differ & large).float().sum().item() / large.float().sum().item() * 1e6:.1f} ppm of those above 128 units')
+    assert (differ & large).float().sum().item() / large.float().sum().item() < 2e-5
+    del hq_default, differ, large
+    rms = exact.double().pow(2).mean().sqrt()
+    diff = (default - exact).abs()
+    worst = (diff.max().double() / rms).item()
+    print(f'[moe] default against exact form at full size: rms difference '
+          f'{(diff.double().pow(2).mean().sqrt() / rms).item():.2e} of the output rms, max {worst:.2e}, '
+          f'{(diff > 1e-2 * rms).float().mean().item() * 1e6:.2f} ppm of the outputs beyond 1e-2')
+    assert worst <= TOL
+    del default
 
-    # the same layer through the weight-streaming GEMMs (gate/up on the bf16 matrix core): same integer stages;
-    # h codes differ only where fp32 is undecided; such a difference on a large element still moves single
-    # outputs by a few percent of the rms, so the whole outputs are compared by their rms difference and by
-    # the share of outputs beyond the tolerance
+    # the same layer through the weight-streaming GEMMs (gate/up on the bf16 matrix core as well): same integer
+    # stages; h codes differ only where fp32 is undecided; such a difference on a large element still moves
+    # single outputs by more than a percent of the rms
     streamed, views_s = run_layer(capi, dts, k, 4, torch.float32)
-    assert (views_s['h_q'].view(torch.uint8) != hq_fixed.view(torch.uint8)).float().mean().item() < 2e-4
-    diff = (streamed - fixed).abs()
+    assert (views_s['h_q'].view(torch.uint8) != hq_exact).float().mean().item() < 2e-4
+    diff = (streamed - exact).abs()
     gap_rms = (diff.double().pow(2).mean().sqrt() / rms).item()
-    beyond = (diff > TOL * rms).float().mean().item()
-    print(f'[moe] tiled + exact pass against streaming form at full size: rms difference {gap_rms:.2e} of the output '
-          f'rms, max {(diff.max().double() / rms).item():.2e}, {beyond * 1e6:.2f} ppm of the outputs beyond {TOL}')
-    assert gap_rms <= 1e-3 and beyond <= 1e-5
+    worst = (diff.max().double() / rms).item()
+    print(f'[moe] tiled exact against streaming form at full size: rms difference {gap_rms:.2e} of the output '
+          f'rms, max {worst:.2e}, {(diff > 1e-2 * rms).float().mean().item() * 1e6:.2f} ppm of the outputs beyond 1e-2')
+    assert gap_rms <= 1e-3 and worst <= TOL
 
 
 def test_rejects_bad_arguments(capi, dev):

@@ -108,8 +108,11 @@ def test_shared_expert_inside_the_routed_launch(capi, dev, shape, config):
     sp, pos, off = moe.sort_pairs(ids, E + 1)
     assert torch.equal(views['sorted_pairs'].cpu(), sp) and torch.equal(views['expert_offsets'].cpu(), off)
     if config:
-        # same GEMM form in both layers: the same tiles are computed and summed in the same order
-        assert torch.equal(fused, run_shared(capi, dts, k, config, torch.float32))
+        # same GEMM form in both layers: the same tiles are computed and summed in the same order (the magnitude
+        # from which the tiled gate/up GEMM repairs its codes follows inter * top_k, which differs between the
+        # two layers, so it is pinned: config bits 12-15)
+        pinned = config | (5 << 12)
+        assert torch.equal(run_fused(capi, dts, k, pinned)[0], run_shared(capi, dts, k, pinned, torch.float32))
     ref = moe.moe_forward_shared(x, logits, *w, *sw, top_k=k, out_dtype=torch.float32)
     rms = ref.double().pow(2).mean().sqrt()
     diff = (fused.cpu() - ref).double().abs()

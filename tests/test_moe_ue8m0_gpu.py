@@ -120,9 +120,9 @@ def test_layer(capi, dev, shape, config):
 @pytest.mark.parametrize('config', [16 | 256, 4])
 @pytest.mark.parametrize('shape', [(300, 512, 256, 4, 2), (520, 768, 384, 3, 3)])
 def test_layer_with_exact_requantisation(capi, dev, shape, config):
-    # the forms whose h agrees with an fp32 evaluation: tiled GEMMs followed by the exact requantisation pass
-    # (config bit 256) and streaming GEMMs (gate/up on the bf16 matrix core): the scales are the oracle's, the
-    # codes differ only where fp32 is undecided, the output meets the plain end-to-end bound
+    # the forms whose h agrees with an fp32 evaluation: tiled GEMMs with gate/up on the bf16 matrix core
+    # (config bit 256) and streaming GEMMs (gate/up on the bf16 matrix core as well): the scales are the oracle's,
+    # the codes differ only where fp32 is undecided, the output meets the plain end-to-end bound
     T, H, I, E, k = shape
     x, logits, w, dts = make_case(dev, T, H, I, E, 70 + T)
     ref, mid = moe.moe_forward(x, logits, *w, top_k=k, out_dtype=torch.float32, return_intermediates=True,
