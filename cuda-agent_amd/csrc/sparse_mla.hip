@@ -1063,7 +1063,6 @@ __global__ __launch_bounds__(256) void sparse_mla_merge_kernel(const PART* __res
     const int lane = threadIdx.x & 63;
     int hg = blockIdx.x;
     int b = blockIdx.y;
-#ifndef MLA_MERGE_PLAIN_MAP
     // request b on XCD b % 8, where the split kernel wrote its partials (see there)
     if ((gridDim.y & 7) == 0) {
         const int linear = blockIdx.x + gridDim.x * blockIdx.y;
@@ -1071,7 +1070,6 @@ __global__ __launch_bounds__(256) void sparse_mla_merge_kernel(const PART* __res
         hg = j % (int)gridDim.x;
         b = (linear & 7) + 8 * (j / (int)gridDim.x);
     }
-#endif
     const int h = hg * 4 + (threadIdx.x >> 6);
     const size_t base = (size_t)b * n_splits * n_heads + h;
     floatx8 o = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -1082,12 +1080,8 @@ __global__ __launch_bounds__(256) void sparse_mla_merge_kernel(const PART* __res
         for (int j = 0; j < BATCH; ++j) {
             // (splits past the end repeat the last one; their weight is 0)
             const int s = s0 + j < n_splits ? s0 + j : n_splits - 1;
-#ifdef MLA_MERGE_PLAIN_LOADS
-            rows[j] = *(reinterpret_cast<const partx8*>(o_part + (base + (size_t)s * n_heads) * D_V) + lane);
-#else
             rows[j] = __builtin_nontemporal_load(
                 reinterpret_cast<const partx8*>(o_part + (base + (size_t)s * n_heads) * D_V) + lane);
-#endif
         }
     };
     // the first rows are requested before anything depends on the log-sum-exps

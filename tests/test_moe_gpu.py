@@ -543,12 +543,14 @@ def test_workspace_binding_at_the_workload_sizes():
     assert 'binding == C ABI at 64 tokens' in out.stdout and 'binding == C ABI at 8192 tokens' in out.stdout
 
 
-def test_workspace_verification_flow():
-    """`python3 -m utils.verification` from inside the workspace, as its user runs it (reduced
-    layer: the full one spends minutes drawing 11 GB of weights on the host)."""
+@pytest.mark.parametrize('config', ['small', '2', '4'])
+def test_workspace_verification_flow(config):
+    """`python3 -m utils.verification` from inside the workspace, as its user runs it: the reduced layer, and the
+    decode and prefill workloads at their full sizes (configs[2] and configs[4]: 256 experts, 11.3 GB of weights,
+    drawn from raw random bits on the GPU)."""
     ws = Path(__file__).resolve().parent.parent / 'cuda-agent_amd' / 'workspaces' / 'moe_fp8'
     assert (ws / 'cuda_extension.so').exists(), 'workspace extension not built'
-    env = dict(os.environ, MOE_CONFIG='small')
+    env = dict(os.environ, MOE_CONFIG=config)
     out = subprocess.run([sys.executable, '-m', 'utils.verification'], cwd=ws, env=env,
                          capture_output=True, text=True, timeout=900)
     assert out.returncode == 0, out.stdout + out.stderr
