@@ -599,10 +599,15 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
         uint16_t* s_near = reinterpret_cast<uint16_t*>(s_sgmax + 4 * TILE_PAIRS);  // [256 pairs][4 row groups][2 halves]
         uint16_t* s_cand = s_near + 8 * TILE_PAIRS;
         float* s_scale = reinterpret_cast<float*>(s_cand + 8 * TILE_PAIRS);      // [256 pairs]
-        int* s_list = reinterpret_cast<int*>(s_scale + TILE_PAIRS);              // [256]
-        int* s_count = s_list + TILE_PAIRS;
-        static_assert(18 * TILE_PAIRS * sizeof(float) + 16 * TILE_PAIRS * sizeof(uint16_t) + TILE_PAIRS * CODE_ROW + 16 <=
-                          2 * STAGE_BYTES, "epilogue LDS");
+        int* s_token = reinterpret_cast<int*>(s_scale + TILE_PAIRS);             // [256] token of a listed pair
+        float* s_tau = reinterpret_cast<float*>(s_token + TILE_PAIRS);           // [256] relative uncertainty of the scale
+        int* s_count = reinterpret_cast<int*>(s_tau + TILE_PAIRS);               // items listed
+        constexpr int MAX_ITEMS = 8192;  // items beyond it (a tile with that many marks) stay unrepaired
+        uint16_t* s_items = reinterpret_cast<uint16_t*>(s_count + 4);            // [MAX_ITEMS] pair << 7 | column
+        static_assert(19 * TILE_PAIRS * sizeof(float) + 16 * TILE_PAIRS * sizeof(uint16_t) + TILE_PAIRS * CODE_ROW + 16 +
+                              MAX_ITEMS * sizeof(uint16_t) <= 2 * STAGE_BYTES, "epilogue LDS");
+        // column, within the group of 128, of bit `bit` of a lane's mark mask number `part` (= 2 * row group + half)
+        auto mark_column = [](int part, int bit) { return (part >> 1) * 32 + 8 * (bit >> 2) + 4 * (part & 1) + (bit & 3); };
         if constexpr (FIX) {
             if (threadIdx.x == 0) *s_count = 0;
         }
@@ -680,8 +685,9 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
             if constexpr (FIX) {
                 s_near[pl * 8 + rg * 2 + half] = (uint16_t)near_bits;
                 s_cand[pl * 8 + rg * 2 + half] = (uint16_t)cand_bits;
-                if (rg == 0 && half == 0) s_scale[pl] = scale;
-            } else if (rg == 0 && half == 0 && pl < cnt) {
+                if (rg == 0 && half == 0) s_scale[pl] = scale, s_tau[pl] = dh_max / fmaxf(m, AMAX_FLOOR);
+            }
+            if (rg == 0 && half == 0 && pl < cnt) {
                 const size_t pos = (size_t)begin + pl;
                 h_s[pos * (inter / GROUP) + rb] = scale;
                 hs_t[(size_t)rb * scale_stride + pos] = scale;
@@ -689,84 +695,95 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
         }
         __syncthreads();
         if constexpr (FIX) {
-            // Exact requantisation of the marked elements. The pairs that hold one are listed; the wavefronts take
-            // them in turn and recompute, as fp32 products of the codes summed in fp64 (the dot product itself
-            // to fp32 accuracy), first the elements that may be the pair's maximum over these 128 columns, which
-            // fixes the scale, then the marked elements, whose codes replace the staged ones. A recomputed element
-            // reads its activation row and its two weight rows (3 K bytes) once more, the weight rows from the L2
-            // this workgroup has just streamed them through.
+            // Exact requantisation of the marked elements: a list of (pair, column) items that the wavefronts take
+            // in turn. An item is recomputed by one wavefront as fp32 products of the codes summed in fp64 (the dot
+            // product itself to fp32 accuracy), all of its loads in flight at once: the activation row and the two
+            // weight rows (3 K bytes) and the block scales. The pair keeps the scale the matrix core's maximum gave
+            // it (off by about 1e-5 of itself, which moves no dequantised value by more than that); the code is the
+            // rounding of exact value / that scale unless the exact scale, which may differ by the relative amount
+            // s_tau, could give another code: only then the elements that may be the pair's maximum are recomputed as
+            // well and the code is taken with the exact scale (a power-of-two scale does not move with the maximum's
+            // 5th digit, so that form never does this).
             if (threadIdx.x < TILE_PAIRS) {
                 const int pl = threadIdx.x;
-                const intx4 nm = *reinterpret_cast<const intx4*>(s_near + pl * 8);
-                if (pl < cnt && (nm[0] | nm[1] | nm[2] | nm[3]) != 0) s_list[atomicAdd(s_count, 1)] = pl;
+                const uint16_t* masks = s_near + pl * 8;
+                const intx4 nm = *reinterpret_cast<const intx4*>(masks);
+                if (pl < cnt && (nm[0] | nm[1] | nm[2] | nm[3]) != 0) {
+                    s_token[pl] = sorted_pairs[(size_t)begin + pl] / top_k;
+                    int n = 0;
+                    for (int part = 0; part < 8; ++part) n += __builtin_popcount(masks[part]);
+                    int slot = atomicAdd(s_count, n);
+                    for (int part = 0; part < 8; ++part) {
+                        for (uint32_t m = masks[part]; m != 0; m &= m - 1) {
+                            if (slot < MAX_ITEMS) s_items[slot] = (uint16_t)((pl << 7) | mark_column(part, __builtin_ctz(m)));
+                            ++slot;
+                        }
+                    }
+                }
             }
             __syncthreads();
-            const int n_list = *s_count;
             const int n_chunks = K / 16;
-            for (int it = wave; it < n_list; it += 8) {
-                const int pl = __builtin_amdgcn_readfirstlane(s_list[it]);
-                const size_t pos = (size_t)begin + pl;
-                const uint8_t* x_row = a_q + (size_t)(sorted_pairs[pos] / top_k) * K;
-                const float* xs = as_t + pos;  // [kb * scale_stride]
-                const uint8_t* gate_rows = w_q + ((size_t)e * n_rows + rb * GROUP) * K;
-                auto exact_h = [&](int col) {  // h of column col of the group (every lane returns the same value)
-                    const uint8_t* gate_row = gate_rows + (size_t)col * K;
-                    const uint8_t* up_row = gate_row + (size_t)inter * K;
-                    double g = 0.0, u = 0.0;
-                    for (int c0 = 0; c0 < n_chunks; c0 += 256) {
-                        intx4 xq[4], wg[4], wu[4];
-                        float sg[4], su[4];
+            const uint8_t* gate_rows = w_q + ((size_t)e * n_rows + rb * GROUP) * K;
+            auto exact_h = [&](int pl, int col) {  // every lane returns the same value
+                const uint8_t* x_row = a_q + (size_t)s_token[pl] * K;
+                const float* xs = as_t + begin + pl;  // [kb * scale_stride]
+                const uint8_t* gate_row = gate_rows + (size_t)col * K;
+                const uint8_t* up_row = gate_row + (size_t)inter * K;
+                double g = 0.0, u = 0.0;
+                for (int c0 = 0; c0 < n_chunks; c0 += 512) {
+                    intx4 xq[8], wg[8], wu[8];
+                    float sg[8], su[8];
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            const int c = c0 + 64 * j + lane;
-                            xq[j] = wg[j] = wu[j] = intx4{0, 0, 0, 0};
-                            sg[j] = su[j] = 0.f;
-                            if (c < n_chunks) {
-                                xq[j] = *reinterpret_cast<const intx4*>(x_row + 16 * c);
-                                wg[j] = *reinterpret_cast<const intx4*>(gate_row + 16 * c);
-                                wu[j] = *reinterpret_cast<const intx4*>(up_row + 16 * c);
-                                const float x_scale = xs[(size_t)(c >> 3) * scale_stride];
-                                sg[j] = x_scale * ws0[c >> 3];
-                                su[j] = x_scale * ws1[c >> 3];
+                    for (int j = 0; j < 8; ++j) {
+                        const int c = c0 + 64 * j + lane;
+                        xq[j] = wg[j] = wu[j] = intx4{0, 0, 0, 0};
+                        sg[j] = su[j] = 0.f;
+                        if (c < n_chunks) {
+                            xq[j] = *reinterpret_cast<const intx4*>(x_row + 16 * c);
+                            wg[j] = *reinterpret_cast<const intx4*>(gate_row + 16 * c);
+                            wu[j] = *reinterpret_cast<const intx4*>(up_row + 16 * c);
+                            sg[j] = xs[(size_t)(c >> 3) * scale_stride];
+                            su[j] = ws1[c >> 3];
+                            const float wsg = ws0[c >> 3];
+                            su[j] *= sg[j];
+                            sg[j] *= wsg;
+                        }
+                    }
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        g += (double)(dot16(xq[j], wg[j]) * sg[j]);
+                        u += (double)(dot16(xq[j], wu[j]) * su[j]);
+                    }
+                }
+                const float gf = (float)wave_sum(g);
+                const float uf = (float)wave_sum(u);
+                return gf / (1.f + expf(-gf)) * uf;
+            };
+            const int n_items = min(*s_count, MAX_ITEMS);
+            for (int it = wave; it < n_items; it += 8) {
+                const int item = __builtin_amdgcn_readfirstlane((int)s_items[it]);
+                const int pl = item >> 7, col = item & 127;
+                const float h = exact_h(pl, col);
+                float scale = s_scale[pl];
+                if constexpr (!UE8M0) {
+                    const float v = fminf(fabsf(h) / scale, E4M3_MAX), tau = v * s_tau[pl];
+                    const int codes = __builtin_amdgcn_cvt_pk_fp8_f32(fmaxf(v - tau, 0.f), fminf(v + tau, E4M3_MAX), 0, false);
+                    if (((codes ^ (codes >> 8)) & 0xff) != 0) {  // (uniform over the wavefront: h is)
+                        float amax = 0.f;
+                        for (int part = 0; part < 8; ++part) {
+                            for (uint32_t cm = __builtin_amdgcn_readfirstlane((uint32_t)s_cand[pl * 8 + part]); cm != 0;
+                                 cm &= cm - 1) {
+                                amax = fmaxf(amax, fabsf(exact_h(pl, mark_column(part, __builtin_ctz(cm)))));
                             }
                         }
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            g += (double)(dot16(xq[j], wg[j]) * sg[j]);
-                            u += (double)(dot16(xq[j], wu[j]) * su[j]);
-                        }
-                    }
-                    const float gf = (float)wave_sum(g);
-                    const float uf = (float)wave_sum(u);
-                    return gf / (1.f + expf(-gf)) * uf;
-                };
-                auto column_of = [&](int part, int bit) { return (part >> 1) * 32 + 8 * (bit >> 2) + 4 * (part & 1) + (bit & 3); };
-                float scale = s_scale[pl];
-                float amax = 0.f;
-                bool any_candidate = false;
-                for (int part = 0; part < 8; ++part) {
-                    for (uint32_t cm = __builtin_amdgcn_readfirstlane((uint32_t)s_cand[pl * 8 + part]); cm != 0; cm &= cm - 1) {
-                        amax = fmaxf(amax, fabsf(exact_h(column_of(part, __builtin_ctz(cm)))));
-                        any_candidate = true;
+                        if (amax > 0.f) scale = group_scale(amax, false);
                     }
                 }
-                if (any_candidate) scale = group_scale(amax, UE8M0);
-                for (int part = 0; part < 8; ++part) {
-                    for (uint32_t nm = __builtin_amdgcn_readfirstlane((uint32_t)s_near[pl * 8 + part]); nm != 0; nm &= nm - 1) {
-                        const int col = column_of(part, __builtin_ctz(nm));
-                        const float v = fminf(fmaxf(exact_h(col) / scale, -E4M3_MAX), E4M3_MAX);
-                        const int code = __builtin_amdgcn_cvt_pk_fp8_f32(v, v, 0, false);
-                        if (lane == 0) s_codes[pl * CODE_ROW + col] = (uint8_t)(code & 0xff);
-                    }
-                }
-                if (lane == 0) s_scale[pl] = scale;
+                const float v = fminf(fmaxf(h / scale, -E4M3_MAX), E4M3_MAX);
+                const int code = __builtin_amdgcn_cvt_pk_fp8_f32(v, v, 0, false);
+                if (lane == 0) s_codes[pl * CODE_ROW + col] = (uint8_t)(code & 0xff);
             }
             __syncthreads();
-            if (threadIdx.x < cnt) {
-                const size_t pos = (size_t)begin + threadIdx.x;
-                h_s[pos * (inter / GROUP) + rb] = s_scale[threadIdx.x];
-                hs_t[(size_t)rb * scale_stride + pos] = s_scale[threadIdx.x];
-            }
         }
         // 8 lanes write the 128 codes of one pair: 8 pairs per instruction, 4 instructions per wavefront
 #pragma unroll

@@ -16,10 +16,17 @@ def both_ways(capi, dev, B, H, N, topk, seed, dtype):
     ws = torch.empty(capi.sparse_mla_workspace_bytes(B, H, topk), dtype=torch.uint8, device=dev)
     capi.sparse_mla_decode_launch(want, q, kv, idx, ws)
     got = torch.full((B, H, 512), float('nan'), dtype=dtype, device=dev)
-    before = torch.cuda.memory_allocated(dev)
+    # a first call may look up the array's address; the call that is watched comes after it. What is watched is the
+    # driver's count of free device memory (an allocation inside the library would not show in torch's allocator).
+    capi.sparse_mla_decode_static_launch(got, q, kv, idx)
+    torch.cuda.synchronize()
+    got.fill_(float('nan'))
+    torch.cuda.synchronize()
+    before, free_before = torch.cuda.memory_allocated(dev), torch.cuda.mem_get_info(dev)[0]
     capi.sparse_mla_decode_static_launch(got, q, kv, idx)
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated(dev) == before
+    assert torch.cuda.mem_get_info(dev)[0] == free_before
     return got, want, (q, kv, idx)
 
 
