@@ -662,6 +662,9 @@ def main():
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run 3 plain device copies of 536 870 912 bytes (a kernel of known traffic, '
                          'for scaling the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)')
+    ap.add_argument('--calibrate-mfma', action=argparse.BooleanOptionalAction, default=True,
+                    help='measure what the matrix cores sustain on random operands, alone and beside an HBM stream '
+                         '(about a second): reported as roofline.sustained_peak')
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py: this build measures one GPU only (no collectives, no sharding); run with --gpus 1')
@@ -738,6 +741,18 @@ def main():
                 achieved=results[k]['roofline']['achieved'], unit=results[k]['roofline']['unit'],
                 steps_timed=results[k]['steps_timed'])
         for k in ('gdn', 'moe_decode', 'mla', 'moe_prefill') if k in results})
+    if args.calibrate_mfma:
+        # measured ceilings next to the data-sheet peaks: a stream of MFMAs on random operands, alone and with half
+        # of every CU's wavefronts streaming 2 GiB from HBM meanwhile (csrc/calibrate.hip)
+        alone, _, _ = capi.calibrate_mfma(0.25, 0, False)
+        beside, tbs, _ = capi.calibrate_mfma(0.25, 2 << 30, False)
+        alone_bf16, _, _ = capi.calibrate_mfma(0.25, 0, True)
+        sustained = dict(e4m3_mfma_alone_pflops=alone, e4m3_mfma_beside_hbm_stream_pflops=beside,
+                         hbm_stream_beside_e4m3_mfma_tbs=tbs, bf16_mfma_alone_pflops=alone_bf16)
+        sustained['note'] = ("calibrate_mfma_launcher: 256 workgroups, 4 wavefronts of each issuing MFMAs on random "
+                             "operands (v_mfma_f32_32x32x64_f8f6f4 / v_mfma_f32_32x32x16_bf16), 4 streaming 16-byte loads; "
+                             "rates over the MFMA loops' own wall-clock ticks, mean of the second half of 0.25 s of launches")
+        line["roofline"]["sustained_peak"] = sustained
     if 'cpu_baseline' in head:
         line["cpu_baseline"] = head['cpu_baseline']
     shown = ('workload', 'value', 'unit', 'ms_per_step', 'dtype', 'roofline', 'cpu_baseline')

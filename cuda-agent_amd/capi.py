@@ -18,6 +18,7 @@ _P = c_void_p
 SIGNATURES = {
     'cuda_agent_amd_last_status': (c_int, []),
     'axpby_launcher': (None, [_P, _P, _P, c_float, c_int, c_int, _P]),
+    'calibrate_mfma_launcher': (None, [_P, _P, c_size_t, _P, _P, c_int, c_int, c_int, _P]),
     'gdn_decode_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int,
                                    c_int, c_int, _P]),
     'gdn_decode_fused_launcher': (None, [_P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int,
@@ -132,6 +133,47 @@ def _device_contiguous(**tensors):
     for name, t in tensors.items():
         _require(t.is_cuda, f'{name} must be a GPU tensor')
         _require(t.is_contiguous(), f'{name} must be contiguous')
+
+
+def calibrate_mfma(seconds=0.25, stream_bytes=0, bf16=False, n_cus=256):
+    """Sustained rate of the matrix cores on random operands, alone or beside an HBM stream: launches the
+    calibration kernel back to back for about ``seconds`` and returns (PFLOP/s over the MFMA loops of the last
+    half of the launches, TB/s streamed beside them, mean kernel time in ms)."""
+    import time
+    import torch
+    dev = torch.device('cuda:0')
+    gen = torch.Generator(device=dev).manual_seed(20270)
+    if bf16:
+        operands = torch.randn(n_cus * 16384 // 2, device=dev, generator=gen).bfloat16()
+    else:
+        operands = (torch.randn(n_cus * 16384, device=dev, generator=gen) * 40).clamp(-448, 448).to(torch.float8_e4m3fn)
+    src = torch.empty(stream_bytes // 4, dtype=torch.int32, device=dev).random_(generator=gen) if stream_bytes else None
+    result = torch.zeros(n_cus, 2, dtype=torch.int64, device=dev)
+    sink = torch.zeros(2, device=dev)
+    iters = 4096
+    flops_per_cu = 4 * iters * 4 * 2 * 32 * 32 * (16 if bf16 else 64)
+
+    def launch():
+        library().calibrate_mfma_launcher(_ptr(operands), _ptr(src) if src is not None else c_void_p(None), stream_bytes,
+                                          _ptr(result), _ptr(sink), n_cus, iters, 1 if bf16 else 0, _stream(None))
+        check_status('calibrate_mfma_launcher')
+
+    t0 = time.perf_counter()
+    rates, streamed, times = [], [], []
+    while time.perf_counter() - t0 < seconds or len(rates) < 4:
+        result.zero_()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        launch()
+        b.record()
+        torch.cuda.synchronize()
+        ticks = result[:, 0].double()
+        rates.append(flops_per_cu * n_cus / (ticks.mean().item() * 1e-8) / 1e15)
+        streamed.append(result[:, 1].sum().item() / (ticks.mean().item() * 1e-8) / 1e12)
+        times.append(a.elapsed_time(b))
+    half = len(rates) // 2
+    mean = lambda v: sum(v[half:]) / len(v[half:])
+    return mean(rates), mean(streamed), mean(times)
 
 
 def axpby_launch(out, a, b, alpha, config=0, stream=None):

@@ -460,6 +460,14 @@ void moe_fp8_fused_shared_launcher(void* out, const void* x, const float* logits
                                    int inter, int n_experts, int top_k, int out_dtype, int config,
                                    hipStream_t stream);
 
+/* Measuring aid of bench.py, no counterpart in the reference workspace: one workgroup per CU whose first four
+ * wavefronts issue `iters` rounds of four e4m3 MFMAs (v_mfma_f32_32x32x64_f8f6f4; config 1: bf16,
+ * v_mfma_f32_32x32x16_bf16) on the random operands given, while the other four stream stream_src (stream_bytes
+ * of it, 0 for none) from memory until the MFMAs are done. result [n_cus][2] uint64, cleared by the caller:
+ * ticks at 100 MHz of each workgroup's MFMA loop, and the bytes streamed meanwhile. operands: n_cus * 16384 bytes. */
+void calibrate_mfma_launcher(const void* operands, const void* stream_src, size_t stream_bytes, void* result,
+                             float* sink, int n_cus, int iters, int config, hipStream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
