@@ -138,7 +138,8 @@ struct Workspace {
     float* y;             // [T*k*H] expert outputs, rows in sorted order: fp32 from the streaming down GEMM; from
                           //         the tiled one fp16 of y / y_scale in the first half of the buffer
     float* y_scale;       // [T*k][H/256] power of two above the largest |y| of each run of 256 columns (tiled)
-    int* tile_start;      // [E+1]  first 256-pair tile of every expert (tiled path)
+    int* tile_start;      // [2E+1] first 256-pair tile of every slot of the dispatch order, then the slots' experts
+                          //        (tiled path)
     float* xs_t;          // [H/128][scale_stride] activation scales by sorted position, transposed
     float* hs_t;          // [I/128][scale_stride] the same for h
     int scale_stride;     // pairs rounded up to 256, plus 256 of padding
@@ -171,7 +172,7 @@ inline Workspace carve_workspace(void* base, int tokens, int hidden, int inter, 
     w.h_s = reinterpret_cast<float*>(take(pairs * (inter / GROUP) * 4));
     w.y = reinterpret_cast<float*>(take(pairs * hidden * 4));
     w.scale_stride = (int)(align_up(pairs, 256) + 256);
-    w.tile_start = reinterpret_cast<int*>(take(((size_t)n_experts + 1) * 4));
+    w.tile_start = reinterpret_cast<int*>(take((2 * (size_t)n_experts + 1) * 4));
     w.xs_t = reinterpret_cast<float*>(take((size_t)(hidden / GROUP) * w.scale_stride * 4));
     w.hs_t = reinterpret_cast<float*>(take((size_t)(inter / GROUP) * w.scale_stride * 4));
     w.y_scale = reinterpret_cast<float*>(take(pairs * ((hidden + 255) / 256) * 4));
