@@ -90,21 +90,20 @@ inline float requant_error_coefficient(int config) {
 }
 
 #ifdef __HIPCC__
-// Marks of one element of h for the exact requantisation. h = sg * u is the element as computed (sg = silu(g)),
-// scale / amax the group's scale and maximum as computed, err the error bound of g and of u, dh_max a bound of
-// the error of any element of the group, scale_uncertain whether the exact maximum may give another scale.
-__device__ __forceinline__ uint32_t requant_marks(float h, float sg, float u, float scale, float amax, float err,
-                                                  float dh_max, bool scale_uncertain, float v_min = 0.f) {
+// Marks of one element of h for the exact requantisation, everything in units of the group's scale (code units):
+// v = |h| / scale as computed, sg = silu(g) and u as computed, err_s the error bound of g and of u, dh_max_s a bound
+// of the error of any element of the group (both divided by the scale), tau_s the relative amount by which the
+// exact scale may differ (0 if it cannot), v_min the magnitude below which an element is not repaired.
+__device__ __forceinline__ uint32_t requant_marks(float v, float sg, float u, float err_s, float dh_max_s, float tau_s,
+                                                  bool scale_uncertain, float v_min) {
     // |d silu / d g| <= 1.1
-    const float dh = (1.1f * fabsf(u) + fabsf(sg)) * err;
-    const float v = fminf(fabsf(h) / scale, E4M3_MAX);
-    // the exact scale differs from `scale` by at most dh_max / amax of itself
-    const float tau = dh / scale + (scale_uncertain ? v * (dh_max / amax) : 0.f);
+    const float tau = fmaf(fmaf(1.1f, fabsf(u), fabsf(sg)), err_s, v * tau_s);
     const float lo = fmaxf(v - tau, 0.f);
     const float hi = fminf(v + tau, E4M3_MAX);
     const int codes = __builtin_amdgcn_cvt_pk_fp8_f32(lo, hi, 0, false);
     uint32_t m = ((codes ^ (codes >> 8)) & 0xff) != 0 && hi >= v_min ? MARK_NEAR : 0u;
-    if (scale_uncertain && fabsf(h) + 2.f * dh_max >= amax) m |= MARK_CANDIDATE;
+    // (the group's maximum has v = 448 by construction)
+    if (scale_uncertain && v + 2.f * dh_max_s >= E4M3_MAX) m |= MARK_CANDIDATE;
     return m;
 }
 #endif

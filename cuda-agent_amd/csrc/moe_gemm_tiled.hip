@@ -702,8 +702,9 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
                     if constexpr (FIX) {
                         const float sg = silu(v);
                         v = sg * acc[1][b][4 * qd + r];
-                        const uint32_t marks = requant_marks(v, sg, acc[1][b][4 * qd + r], scale, fmaxf(m, AMAX_FLOOR), err,
-                                                             dh_max, uncertain, v_min);
+                        const uint32_t marks = requant_marks(fminf(fabsf(v) * inv_scale, E4M3_MAX), sg, acc[1][b][4 * qd + r],
+                                                             err * inv_scale, dh_max * inv_scale,
+                                                             uncertain ? dh_max / fmaxf(m, AMAX_FLOOR) : 0.f, uncertain, v_min);
                         near_bits |= (marks & MARK_NEAR ? 1u : 0u) << (4 * qd + r);
                         cand_bits |= (marks & MARK_CANDIDATE ? 1u : 0u) << (4 * qd + r);
                     }
@@ -762,28 +763,31 @@ __global__ __launch_bounds__(512) void moe_tiled_gemm_kernel(
                 const uint8_t* up_row = gate_row + (size_t)inter * K;
                 double g = 0.0, u = 0.0;
                 for (int c0 = 0; c0 < n_chunks; c0 += 512) {
+                    // (a load instruction costs a wavefront 150-300 cycles to issue whatever it fetches: the scale
+                    // products of the 64 K blocks of this stretch are fetched by one lane each, three loads, and
+                    // handed to the lanes that need them by shuffles, instead of three loads per 1 KB of a row)
+                    const int kb = (c0 >> 3) + lane;
+                    float sg_kb = 0.f, su_kb = 0.f;
+                    if (kb < KB) {
+                        const float x_scale = xs[(size_t)kb * scale_stride];
+                        sg_kb = x_scale * ws0[kb];
+                        su_kb = x_scale * ws1[kb];
+                    }
                     intx4 xq[8], wg[8], wu[8];
-                    float sg[8], su[8];
 #pragma unroll
                     for (int j = 0; j < 8; ++j) {
                         const int c = c0 + 64 * j + lane;
                         xq[j] = wg[j] = wu[j] = intx4{0, 0, 0, 0};
-                        sg[j] = su[j] = 0.f;
                         if (c < n_chunks) {
                             xq[j] = *reinterpret_cast<const intx4*>(x_row + 16 * c);
                             wg[j] = *reinterpret_cast<const intx4*>(gate_row + 16 * c);
                             wu[j] = *reinterpret_cast<const intx4*>(up_row + 16 * c);
-                            sg[j] = xs[(size_t)(c >> 3) * scale_stride];
-                            su[j] = ws1[c >> 3];
-                            const float wsg = ws0[c >> 3];
-                            su[j] *= sg[j];
-                            sg[j] *= wsg;
                         }
                     }
 #pragma unroll
                     for (int j = 0; j < 8; ++j) {
-                        g += (double)(dot16(xq[j], wg[j]) * sg[j]);
-                        u += (double)(dot16(xq[j], wu[j]) * su[j]);
+                        g += (double)(dot16(xq[j], wg[j]) * __shfl(sg_kb, 8 * j + (lane >> 3)));
+                        u += (double)(dot16(xq[j], wu[j]) * __shfl(su_kb, 8 * j + (lane >> 3)));
                     }
                 }
                 const float gf = (float)wave_sum(g);
