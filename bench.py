@@ -33,24 +33,24 @@ HBM_PEAK_GBS = 8000.0
 FP8_PEAK_TFLOPS = 5033.0
 METRIC = "GB/s & % HBM peak (GDN/MoE/MLA decode); fp8 TFLOP/s % MFMA peak (MoE prefill)"
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled
+# HBM bytes per step (summed over the workload's kernels) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled
 # by the same counters read on a plain 512 MiB copy kernel (FETCH_SIZE x 1.99986, WRITE_SIZE x 1,
-# both in KiB); the counter summary is profiles/all_workloads_hbm_traffic_pmc.md.
-# None = not measured.
-# Stamp: taken from the library as built from the sources of this tree (fp16 expert outputs in the prefill down
-# GEMM, bf16 matrix core in the decode gate/up GEMM); a change to a kernel's data movement needs a new run of
-# the two commands in that file.
-MEASURED_TRAFFIC = {'gdn': 1085846000, 'moe_decode': 6664690000, 'mla': 196017000, 'index_scores': 553927000,
-                    'index_scores_fp8': 289777000, 'moe_prefill': 11426305000, 'mla_fp8_cache': 145212000,
+# both in KiB); the counter summary is profiles/all_workloads_hbm_traffic_pmc.md, whose "HBM bytes" column
+# holds each of these figures (a test checks that). None = not measured.
+# Stamp: taken from the library as built from the sources of this tree; a change to a kernel's data movement needs
+# a new run of the two commands in that file.
+MEASURED_TRAFFIC = {'gdn': 1085858000, 'moe_decode': 10002073000, 'mla': 238270000, 'index_scores': 553927000,
+                    'index_scores_fp8': 289777000, 'moe_prefill': 22426952000, 'mla_fp8_cache': 187610000,
                     'topk_select': 9216000}
 # Matrix-pipe occupancy of the dominant kernels from rocprofv3 --pmc (SQ_VALU_MFMA_BUSY_CYCLES over 1024 SIMDs x
 # GRBM_GUI_ACTIVE cycles per XCD, the timed launches of bench.py's own loop; the derived MfmaUtil counter reads
-# 39.6 / 33.5 / 22.9 %) and the clock by GRBM_GUI_ACTIVE / 8 / duration in the same run; the summary is
-# profiles/moe_prefill_mla_matrix_core_counters_pmc.md. Measured figures of that run, not of this one.
+# 33.3 / 33.7 / 23.5 %) and the clock by GRBM_GUI_ACTIVE / 8 / duration in the same run (SQ_BUSY_CU_CYCLES / 256 /
+# duration for the short sparse-MLA kernel); the summary is profiles/moe_prefill_mla_matrix_core_counters_pmc.md.
+# Measured figures of that run, not of this one.
 MEASURED_MFMA = {
-    'moe_prefill': dict(mfma_busy=0.415, clock_ghz=1.92, kernel='moe_tiled_gemm_kernel<true> (gate/up)',
-                        mfma_busy_down=0.351, clock_ghz_down=1.75),
-    'mla': dict(mfma_busy=0.238, clock_ghz=2.03, kernel='sparse_mla_split8_kernel<false>'),
+    'moe_prefill': dict(mfma_busy=0.343, clock_ghz=1.97, kernel='moe_tiled_gemm_kernel<true> (gate/up)',
+                        mfma_busy_down=0.345, clock_ghz_down=1.84),
+    'mla': dict(mfma_busy=0.241, clock_ghz=2.05, kernel='sparse_mla_split8_kernel<false>'),
 }
 
 

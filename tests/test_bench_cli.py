@@ -58,9 +58,15 @@ def test_measured_constants_of_bench_are_the_figures_of_the_committed_profiles()
             values[node.targets[0].id] = ast.literal_eval(ast.unparse(node.value).replace('dict(', 'dict(')) \
                 if node.targets[0].id == 'MEASURED_TRAFFIC' else ast.unparse(node.value)
     traffic_md = (REPO / 'profiles' / 'all_workloads_hbm_traffic_pmc.md').read_text()
+    # the fourth column of the summary's table ("HBM bytes (scaled)") of some row, not just any place in the file
+    hbm_bytes = set()
+    for row in traffic_md.splitlines():
+        cells = [c.strip() for c in row.split('|')]
+        if row.startswith('|') and len(cells) >= 6 and re.fullmatch(r'[\d ]+', cells[4] or 'x'):
+            hbm_bytes.add(int(cells[4].replace(' ', '')))
+    assert len(hbm_bytes) >= 8
     for name, nbytes in values['MEASURED_TRAFFIC'].items():
-        spaced = f'{nbytes:,}'.replace(',', ' ')
-        assert spaced in traffic_md, (name, spaced)
+        assert nbytes in hbm_bytes, (name, nbytes)
     counters_md = (REPO / 'profiles' / 'moe_prefill_mla_matrix_core_counters_pmc.md').read_text()
     for figure in re.findall(r'mfma_busy(?:_down)?=([0-9.]+)', values['MEASURED_MFMA']):
         assert figure in counters_md, figure
