@@ -106,3 +106,25 @@ def test_router_chain(capi, dev, seed):
     same = (ids.cpu() == want_ids).all(dim=1)
     assert (~same).sum().item() <= max(1, T // 500)
     torch.testing.assert_close(wts.cpu()[same], want_w[same], rtol=1e-5, atol=1e-9)
+
+
+@pytest.mark.parametrize('seed', range(8))
+def test_moe_layer(capi, dev, seed):
+    """The whole layer on a random valid shape, stage by stage and end to end (test_moe_gpu.check_layer states the
+    bars): the streaming GEMMs, and the tiled ones (config bit 16) both with gate/up on the bf16 matrix core and as
+    the layer runs them by default, e4m3 matrix core with the large codes repaired."""
+    from test_moe_gpu import check_layer
+    rng = torch.Generator().manual_seed(9000 + seed)
+    T = _pick(rng, [1, 7, 33, 129, 300, 517])
+    form = seed % 3
+    H = 128 * _pick(rng, [1, 2, 3, 6]) if form == 0 else 256 * _pick(rng, [1, 2, 3])   # (the tiled GEMMs: multiples of 256)
+    inter = 128 * _pick(rng, [1, 2, 4])
+    E = _pick(rng, [2, 3, 5, 8])
+    k = int(torch.randint(1, min(E, 4) + 1, (1,), generator=rng))
+    biased = [0] if seed % 2 else None
+    if form == 0:
+        check_layer(capi, dev, T, H, inter, E, k, 9100 + seed, config=1, biased=biased)
+    elif form == 1:
+        check_layer(capi, dev, T, H, inter, E, k, 9100 + seed, config=16, biased=biased, requant='exact')
+    else:
+        check_layer(capi, dev, T, H, inter, E, k, 9100 + seed, config=16, biased=biased, requant='repaired')
