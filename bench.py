@@ -749,6 +749,10 @@ def main():
         alone_bf16, _, _ = capi.calibrate_mfma(0.25, 0, True)
         sustained = dict(e4m3_mfma_alone_pflops=alone, e4m3_mfma_beside_hbm_stream_pflops=beside,
                          hbm_stream_beside_e4m3_mfma_tbs=tbs, bf16_mfma_alone_pflops=alone_bf16)
+        # the clock the matrix pipes run at against the share of the chip that is busy: the same loop (which keeps
+        # every SIMD's pipe full: 8192 flops per CU and cycle) on 32, 128 and all 256 CUs
+        sustained['e4m3_mfma_clock_ghz_by_busy_cus'] = {
+            str(n): capi.calibrate_mfma(0.15, 0, False, n)[0] * 1e6 / (n * 8192) for n in (32, 128, 256)}
         sustained['note'] = ("calibrate_mfma_launcher: 256 workgroups, 4 wavefronts of each issuing MFMAs on random "
                              "operands (v_mfma_f32_32x32x64_f8f6f4 / v_mfma_f32_32x32x16_bf16), 4 streaming 16-byte loads; "
                              "rates over the MFMA loops' own wall-clock ticks, mean of the second half of 0.25 s of launches")
